@@ -1,0 +1,104 @@
+// Shared device helpers for the gfx950 kernels: 16-bit element traits, MFMA
+// wrappers, wave64 shuffles, error plumbing for the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/fsa_hip.h"
+
+namespace fsa {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVE = 64;
+constexpr float LOG2E = 1.4426950408889634f;
+
+// ---- element traits -------------------------------------------------------
+template <typename T> struct Elem;
+
+template <> struct Elem<__bf16> {
+  typedef bf16x8 vec8;
+  typedef bf16x4 vec4;
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <> struct Elem<_Float16> {
+  typedef f16x8 vec8;
+  typedef f16x4 vec4;
+  static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// 16-byte / 8-byte raw moves (global or LDS) reinterpreted as element vectors.
+template <typename V> __device__ __forceinline__ V load16(const void* p) {
+  uint4 r = *reinterpret_cast<const uint4*>(p);
+  return __builtin_bit_cast(V, r);
+}
+template <typename V> __device__ __forceinline__ void store16(void* p, V v) {
+  *reinterpret_cast<uint4*>(p) = __builtin_bit_cast(uint4, v);
+}
+template <typename V> __device__ __forceinline__ V load8(const void* p) {
+  uint2 r = *reinterpret_cast<const uint2*>(p);
+  return __builtin_bit_cast(V, r);
+}
+template <typename V> __device__ __forceinline__ void store8(void* p, V v) {
+  *reinterpret_cast<uint2*>(p) = __builtin_bit_cast(uint2, v);
+}
+
+template <typename T> __device__ __forceinline__ typename Elem<T>::vec8 zero8() {
+  uint4 z = make_uint4(0, 0, 0, 0);
+  return __builtin_bit_cast(typename Elem<T>::vec8, z);
+}
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// largest i in [0, n) with a[i] <= x, for ascending a[0..n) with a[0] <= x
+__device__ __forceinline__ int upper_seg(const int32_t* __restrict__ a, int n, int x) {
+  int lo = 0, hi = n;  // invariant a[lo] <= x, a[hi] > x (virtual)
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if (a[mid] <= x) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+// ---- host-side error plumbing --------------------------------------------
+void set_error(const char* fmt, ...);
+
+#define FSA_CHECK_ARG(cond, ...)            \
+  do {                                      \
+    if (!(cond)) {                          \
+      fsa::set_error(__VA_ARGS__);          \
+      return FSA_ERR_INVALID;               \
+    }                                       \
+  } while (0)
+
+#define FSA_CHECK_LAUNCH(what)                                               \
+  do {                                                                       \
+    hipError_t e__ = hipGetLastError();                                      \
+    if (e__ != hipSuccess) {                                                 \
+      fsa::set_error("%s: %s", what, hipGetErrorString(e__));                \
+      return (int)e__;                                                       \
+    }                                                                        \
+  } while (0)
+
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+}  // namespace fsa

@@ -1,0 +1,338 @@
+// Inverted block->query index for selected attention (gfx950).
+//
+// The (query, slot) entries of topk_idx are keyed by global block id and put
+// through a stable LSD radix sort (8-bit digits, wave64 ballot ranking), so
+// that inside every block the queries appear in ascending order - the order the
+// reference obtains by compacting a dense [nblk, N] table
+// (fsa/ops/FSA_topk_sparse_attention.py:1016).  Work and memory are linear in
+// N*T; nothing of size nblk*N is ever materialised.
+#include "fsa_common.h"
+
+namespace fsa {
+
+constexpr int RS_THREADS = 256;
+constexpr int RS_WAVES = RS_THREADS / WAVE;
+constexpr int RS_ROUNDS = 8;
+constexpr int RS_PER_WAVE = RS_ROUNDS * WAVE;   // 512 consecutive items per wave
+constexpr int RS_TILE = RS_WAVES * RS_PER_WAVE; // 2048 items per work-group
+constexpr int SCAN_THREADS = 1024;
+
+// Exclusive scan of one int per thread over a SCAN_THREADS-wide block.
+__device__ __forceinline__ int block_exclusive_scan(int v, int* total) {
+  __shared__ int wave_sums[SCAN_THREADS / WAVE];
+  __shared__ int block_total;
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  int inc = v;
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    int t = __shfl_up(inc, o, WAVE);
+    if (lane >= o) inc += t;
+  }
+  if (lane == WAVE - 1) wave_sums[w] = inc;
+  __syncthreads();
+  if (w == 0) {
+    int s = lane < (int)(blockDim.x / WAVE) ? wave_sums[lane] : 0;
+    int si = s;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+      int t = __shfl_up(si, o, WAVE);
+      if (lane >= o) si += t;
+    }
+    if (lane < (int)(blockDim.x / WAVE)) wave_sums[lane] = si - s;
+    if (lane == WAVE - 1) block_total = si;
+  }
+  __syncthreads();
+  int r = wave_sums[w] + inc - v;
+  *total = block_total;
+  __syncthreads();
+  return r;
+}
+
+__global__ void cu_blocks_kernel(const int32_t* __restrict__ cu_seqlens, int batch, int block_size,
+                                 int32_t* __restrict__ cu_blocks) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    int acc = 0;
+    cu_blocks[0] = 0;
+    for (int s = 0; s < batch; ++s) {
+      int len = cu_seqlens[s + 1] - cu_seqlens[s];
+      acc += (len + block_size - 1) / block_size;
+      cu_blocks[s + 1] = acc;
+    }
+  }
+}
+
+// key = global block id, or `sentinel` for padding / out-of-range ids; val = n*T + t
+__global__ void __launch_bounds__(256)
+make_keys_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
+                 const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ cu_blocks,
+                 int batch, int64_t n_items, int topk, uint32_t sentinel,
+                 uint32_t* __restrict__ keys, uint32_t* __restrict__ vals) {
+  const int h = blockIdx.y;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_items) return;
+  const int token = (int)(idx / topk);
+  const int t = (int)(idx - (int64_t)token * topk);
+  const int b = topk_idx[h * stride_h + (int64_t)token * stride_n + t];
+  const int s = upper_seg(cu_seqlens, batch, token);
+  const int b0 = cu_blocks[s], nb = cu_blocks[s + 1] - b0;
+  keys[h * n_items + idx] = (b >= 0 && b < nb) ? (uint32_t)(b0 + b) : sentinel;
+  vals[h * n_items + idx] = (uint32_t)idx;
+}
+
+// table[h][digit][tile] = number of items of the tile with that digit
+__global__ void __launch_bounds__(RS_THREADS)
+radix_hist_kernel(const uint32_t* __restrict__ keys, int64_t n_items, int shift, int ntiles,
+                  uint32_t* __restrict__ table) {
+  __shared__ uint32_t hist[256];
+  const int h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+  hist[tid] = 0;
+  __syncthreads();
+  const uint32_t* kh = keys + h * n_items;
+#pragma unroll
+  for (int j = 0; j < RS_ROUNDS; ++j) {
+    int64_t idx = (int64_t)tile * RS_TILE + j * RS_THREADS + tid;
+    if (idx < n_items) atomicAdd(&hist[(kh[idx] >> shift) & 255u], 1u);
+  }
+  __syncthreads();
+  table[((int64_t)h * 256 + tid) * ntiles + tile] = hist[tid];
+}
+
+// in-place exclusive scan of table[h][0 .. 256*ntiles)
+__global__ void __launch_bounds__(SCAN_THREADS)
+radix_scan_kernel(uint32_t* __restrict__ table, int ntiles) {
+  const int h = blockIdx.x;
+  const int64_t m = (int64_t)256 * ntiles;
+  uint32_t* t = table + (int64_t)h * m;
+  const int64_t per = (m + SCAN_THREADS - 1) / SCAN_THREADS;
+  const int64_t lo = (int64_t)threadIdx.x * per;
+  const int64_t hi = lo + per < m ? lo + per : m;
+  int sum = 0;
+  for (int64_t i = lo; i < hi; ++i) sum += (int)t[i];
+  int total;
+  int run = block_exclusive_scan(sum, &total);
+  for (int64_t i = lo; i < hi; ++i) {
+    int c = (int)t[i];
+    t[i] = (uint32_t)run;
+    run += c;
+  }
+}
+
+// Stable scatter of one 8-bit digit.  Item order inside a tile is
+// (wave, round, lane), i.e. the original order.
+__global__ void __launch_bounds__(RS_THREADS)
+radix_scatter_kernel(const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
+                     uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
+                     int64_t n_items, int shift, int ntiles, const uint32_t* __restrict__ table) {
+  __shared__ uint32_t cnt[RS_WAVES][256];
+  const int h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1), w = tid / WAVE;
+  for (int i = tid; i < RS_WAVES * 256; i += RS_THREADS) (&cnt[0][0])[i] = 0;
+  __syncthreads();
+  const uint32_t* kh = keys_in + h * n_items;
+  const uint32_t* vh = vals_in + h * n_items;
+  uint32_t key[RS_ROUNDS], val[RS_ROUNDS], rank[RS_ROUNDS];
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+  for (int r = 0; r < RS_ROUNDS; ++r) {
+    const int64_t idx = (int64_t)tile * RS_TILE + w * RS_PER_WAVE + r * WAVE + lane;
+    const bool ok = idx < n_items;
+    key[r] = ok ? kh[idx] : 0u;
+    val[r] = ok ? vh[idx] : 0u;
+    const uint32_t d = (key[r] >> shift) & 255u;
+    uint64_t peers = __ballot(ok);
+#pragma unroll
+    for (int bit = 0; bit < 8; ++bit) {
+      const bool one = (d >> bit) & 1u;
+      const uint64_t b = __ballot(one);
+      peers &= one ? b : ~b;
+    }
+    uint32_t old = 0;
+    if (ok) {
+      old = cnt[w][d];
+      rank[r] = old + (uint32_t)__popcll(peers & lt_mask);
+    } else {
+      rank[r] = 0;
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (ok && (peers & lt_mask) == 0) cnt[w][d] = old + (uint32_t)__popcll(peers);
+    __builtin_amdgcn_wave_barrier();
+  }
+  __syncthreads();
+  {  // per digit: global base of this tile + exclusive prefix over waves
+    const int d = tid;
+    uint32_t run = table[((int64_t)h * 256 + d) * ntiles + tile];
+#pragma unroll
+    for (int ww = 0; ww < RS_WAVES; ++ww) {
+      uint32_t c = cnt[ww][d];
+      cnt[ww][d] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  uint32_t* ko = keys_out + h * n_items;
+  uint32_t* vo = vals_out + h * n_items;
+#pragma unroll
+  for (int r = 0; r < RS_ROUNDS; ++r) {
+    const int64_t idx = (int64_t)tile * RS_TILE + w * RS_PER_WAVE + r * WAVE + lane;
+    if (idx < n_items) {
+      const uint32_t d = (key[r] >> shift) & 255u;
+      const uint32_t dst = cnt[w][d] + rank[r];
+      ko[dst] = key[r];
+      vo[dst] = val[r];
+    }
+  }
+}
+
+__global__ void __launch_bounds__(256)
+finalize_items_kernel(const uint32_t* __restrict__ keys, const uint32_t* __restrict__ vals,
+                      int64_t n_items, int topk, uint32_t sentinel,
+                      int32_t* __restrict__ sel_tokens, int32_t* __restrict__ slot_of) {
+  const int h = blockIdx.y;
+  const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (p >= n_items) return;
+  const uint32_t key = keys[h * n_items + p];
+  const uint32_t val = vals[h * n_items + p];
+  const bool ok = key != sentinel;
+  sel_tokens[h * n_items + p] = ok ? (int32_t)(val / (uint32_t)topk) : -1;
+  slot_of[h * n_items + val] = ok ? (int32_t)p : -1;
+}
+
+// starts[h][gb] = first position whose key >= gb; counts = adjacent difference
+__global__ void __launch_bounds__(256)
+starts_kernel(const uint32_t* __restrict__ keys, int64_t n_items, int64_t max_blocks,
+              int32_t* __restrict__ starts, int32_t* __restrict__ counts) {
+  const int h = blockIdx.y;
+  const int64_t gb = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (gb > max_blocks) return;
+  const uint32_t* kh = keys + h * n_items;
+  auto lower = [&](uint32_t x) {
+    int64_t lo = 0, hi = n_items;
+    while (lo < hi) {
+      int64_t mid = (lo + hi) >> 1;
+      if (kh[mid] < x) lo = mid + 1; else hi = mid;
+    }
+    return (int32_t)lo;
+  };
+  const int32_t s0 = lower((uint32_t)gb);
+  starts[h * (max_blocks + 1) + gb] = s0;
+  if (gb < max_blocks) counts[h * max_blocks + gb] = lower((uint32_t)gb + 1) - s0;
+}
+
+__global__ void __launch_bounds__(SCAN_THREADS)
+tiles_kernel(const int32_t* __restrict__ counts, int64_t max_blocks, int group_size, int rows_per_tile,
+             int32_t* __restrict__ tile_prefix) {
+  const int h = blockIdx.x;
+  const int32_t* c = counts + h * max_blocks;
+  int32_t* tp = tile_prefix + h * (max_blocks + 1);
+  const int64_t per = (max_blocks + SCAN_THREADS - 1) / SCAN_THREADS;
+  const int64_t lo = (int64_t)threadIdx.x * per;
+  const int64_t hi = lo + per < max_blocks ? lo + per : max_blocks;
+  auto ntile = [&](int64_t gb) {
+    return (int)(((int64_t)c[gb] * group_size + rows_per_tile - 1) / rows_per_tile);
+  };
+  int sum = 0;
+  for (int64_t i = lo; i < hi; ++i) sum += ntile(i);
+  int total;
+  int run = block_exclusive_scan(sum, &total);
+  for (int64_t i = lo; i < hi; ++i) {
+    tp[i] = run;
+    run += ntile(i);
+  }
+  if (threadIdx.x == 0) tp[max_blocks] = total;
+}
+
+}  // namespace fsa
+
+using namespace fsa;
+
+static void index_ws_layout(int64_t n_items, int hkv, size_t* off_keys, size_t* off_vals,
+                            size_t* off_table, size_t* total) {
+  const size_t buf = align_up((size_t)n_items * hkv * 4, 256);
+  const int64_t ntiles = (n_items + RS_TILE - 1) / RS_TILE;
+  off_keys[0] = 0;
+  off_keys[1] = buf;
+  off_vals[0] = 2 * buf;
+  off_vals[1] = 3 * buf;
+  *off_table = 4 * buf;
+  *total = 4 * buf + align_up((size_t)hkv * 256 * ntiles * 4, 256);
+}
+
+extern "C" size_t fsa_index_workspace_bytes(int64_t total_tokens, int32_t topk, int32_t num_kv_heads,
+                                            int64_t max_blocks) {
+  (void)max_blocks;
+  size_t ok[2], ov[2], ot, total;
+  index_ws_layout(total_tokens * topk, num_kv_heads, ok, ov, &ot, &total);
+  return total;
+}
+
+extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, int64_t topk_stride_n,
+                               const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                               int32_t num_kv_heads, int32_t topk, int32_t block_size,
+                               int64_t max_blocks, int32_t* cu_blocks, int32_t* counts,
+                               int32_t* starts, int32_t* sel_tokens, int32_t* slot_of,
+                               void* workspace, size_t workspace_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FSA_CHECK_ARG(topk_idx && cu_seqlens && cu_blocks && counts && starts && sel_tokens && slot_of,
+                "fsa_build_index: null pointer");
+  FSA_CHECK_ARG(batch >= 1 && total_tokens >= 1 && num_kv_heads >= 1 && topk >= 1,
+                "fsa_build_index: batch, total_tokens, num_kv_heads and topk must be positive");
+  FSA_CHECK_ARG(block_size >= 1, "fsa_build_index: block_size must be positive");
+  FSA_CHECK_ARG(max_blocks >= 1 && max_blocks < (1 << 24),
+                "fsa_build_index: max_blocks=%lld out of range", (long long)max_blocks);
+  const int64_t n_items = total_tokens * topk;
+  FSA_CHECK_ARG(n_items < ((int64_t)1 << 31), "fsa_build_index: total_tokens*topk must be < 2^31");
+  size_t ok[2], ov[2], ot, total;
+  index_ws_layout(n_items, num_kv_heads, ok, ov, &ot, &total);
+  if (workspace == nullptr || workspace_bytes < total) {
+    set_error("fsa_build_index: workspace too small (%zu < %zu)", workspace_bytes, total);
+    return FSA_ERR_WORKSPACE;
+  }
+  char* ws = (char*)workspace;
+  uint32_t* keys[2] = {(uint32_t*)(ws + ok[0]), (uint32_t*)(ws + ok[1])};
+  uint32_t* vals[2] = {(uint32_t*)(ws + ov[0]), (uint32_t*)(ws + ov[1])};
+  uint32_t* table = (uint32_t*)(ws + ot);
+  const int ntiles = (int)((n_items + RS_TILE - 1) / RS_TILE);
+  const uint32_t sentinel = (uint32_t)max_blocks;
+
+  cu_blocks_kernel<<<1, 64, 0, stream>>>(cu_seqlens, batch, block_size, cu_blocks);
+  dim3 g_items((unsigned)((n_items + 255) / 256), num_kv_heads);
+  make_keys_kernel<<<g_items, 256, 0, stream>>>(topk_idx, topk_stride_h, topk_stride_n, cu_seqlens,
+                                                cu_blocks, batch, n_items, topk, sentinel, keys[0],
+                                                vals[0]);
+  int bits = 1;
+  while (((uint64_t)1 << bits) <= (uint64_t)sentinel) ++bits;
+  const int passes = (bits + 7) / 8;
+  int cur = 0;
+  for (int p = 0; p < passes; ++p) {
+    dim3 g_tiles(ntiles, num_kv_heads);
+    radix_hist_kernel<<<g_tiles, RS_THREADS, 0, stream>>>(keys[cur], n_items, 8 * p, ntiles, table);
+    radix_scan_kernel<<<num_kv_heads, SCAN_THREADS, 0, stream>>>(table, ntiles);
+    radix_scatter_kernel<<<g_tiles, RS_THREADS, 0, stream>>>(keys[cur], vals[cur], keys[cur ^ 1],
+                                                             vals[cur ^ 1], n_items, 8 * p, ntiles,
+                                                             table);
+    cur ^= 1;
+  }
+  finalize_items_kernel<<<g_items, 256, 0, stream>>>(keys[cur], vals[cur], n_items, topk, sentinel,
+                                                     sel_tokens, slot_of);
+  dim3 g_blocks((unsigned)((max_blocks + 1 + 255) / 256), num_kv_heads);
+  starts_kernel<<<g_blocks, 256, 0, stream>>>(keys[cur], n_items, max_blocks, starts, counts);
+  FSA_CHECK_LAUNCH("fsa_build_index");
+  return 0;
+}
+
+extern "C" int fsa_build_tiles(const int32_t* counts, int32_t num_kv_heads, int64_t max_blocks,
+                               int32_t group_size, int32_t rows_per_tile, int32_t* tile_prefix,
+                               void* stream_) {
+  FSA_CHECK_ARG(counts && tile_prefix, "fsa_build_tiles: null pointer");
+  FSA_CHECK_ARG(num_kv_heads >= 1 && max_blocks >= 1 && group_size >= 1 && rows_per_tile >= 1,
+                "fsa_build_tiles: sizes must be positive");
+  tiles_kernel<<<num_kv_heads, SCAN_THREADS, 0, (hipStream_t)stream_>>>(counts, max_blocks, group_size,
+                                                                        rows_per_tile, tile_prefix);
+  FSA_CHECK_LAUNCH("fsa_build_tiles");
+  return 0;
+}
+
+extern "C" int64_t fsa_max_tiles(int64_t total_tokens, int32_t topk, int32_t group_size,
+                                 int32_t rows_per_tile, int64_t max_blocks) {
+  return (total_tokens * topk * group_size + rows_per_tile - 1) / rows_per_tile + max_blocks;
+}

@@ -1,0 +1,390 @@
+// Selected attention forward for gfx950.
+//
+// Stage 1 (selattn_fwd_main_kernel): KV blocks on the outside.  A work-group
+// owns one kv block of one kv head (K and V^T staged in LDS once) and a range
+// of the gathered rows of that block; a row is one (query, head-in-group) pair,
+// so a GQA group of any size fills MFMA tiles without padding.  Each wave takes
+// 32 rows: S^T = K Q^T (32x32x16 MFMA, one row per lane), a single-block
+// softmax in registers, O^T = V^T P^T, and writes the normalised partial row
+// and its base-2 LSE.
+// Stage 2 (selattn_fwd_reduce_kernel): query-major merge of the <= T partials
+// of each (query, head) with shuffles, 16-byte coalesced loads, no atomics.
+//
+// Semantics follow fsa/ops/FSA_topk_sparse_attention.py:382-566 (main),
+// :138-281 (reduce); the causal mask is q_pos >= key_pos (:520) and the LSE is
+// base 2 (:256-261).
+#include "fsa_common.h"
+
+namespace fsa {
+
+struct SelFwdParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  int64_t q_sn, q_sh, k_sn, k_sh, v_sn, v_sh;
+  const int32_t* cu_seqlens;
+  const int32_t* cu_blocks;
+  const int32_t* counts;
+  const int32_t* starts;
+  const int32_t* sel_tokens;
+  const int32_t* tile_prefix;
+  int batch;
+  int64_t max_blocks;
+  int64_t cap;  // N * T: capacity of the per-head pair list
+  int g;
+  float scale_log2;
+  void* o_part;
+  float* lse_part;
+};
+
+constexpr int SEL_THREADS = 256;
+constexpr int SEL_WG_ROWS = 128;                 // rows per pass of the 4 waves
+constexpr int SEL_TILE_ROWS = 4 * SEL_WG_ROWS;   // rows per work-group
+
+template <int D, int BK> struct SelLds {
+  static constexpr int KS = D + 8;   // K row stride in elements (16 B pad: bank spread)
+  static constexpr int VS = BK + 4;  // V^T row stride in elements
+  static constexpr int BYTES = (BK * KS + D * VS) * 2;
+};
+
+template <typename T, int D, int BK>
+__global__ void __launch_bounds__(SEL_THREADS)
+selattn_fwd_main_kernel(SelFwdParams p) {
+  typedef typename Elem<T>::vec8 vec8;
+  typedef typename Elem<T>::vec4 vec4;
+  constexpr int KS = SelLds<D, BK>::KS, VS = SelLds<D, BK>::VS;
+  constexpr int NA = BK / 32;   // S^T accumulators (32 keys each)
+  constexpr int NKS = D / 16;   // k-steps of QK^T
+  constexpr int NDT = D / 32;   // O^T accumulators (32 dims each)
+  constexpr int NJ = BK / 16;   // k-steps of PV
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* Ks = reinterpret_cast<T*>(smem);
+  T* Vt = Ks + BK * KS;
+
+  const int h = blockIdx.y;
+  const int64_t nbp1 = p.max_blocks + 1;
+  const int32_t* tp = p.tile_prefix + h * nbp1;
+  const int w = blockIdx.x;
+  if (w >= tp[p.max_blocks]) return;
+  const int gb = upper_seg(tp, (int)p.max_blocks, w);
+  const int s = upper_seg(p.cu_blocks, p.batch, gb);
+  const int b_local = gb - p.cu_blocks[s];
+  const int seq_start = p.cu_seqlens[s], seq_end = p.cu_seqlens[s + 1];
+  const int tok0 = seq_start + b_local * BK;
+  const int rows = p.counts[h * p.max_blocks + gb] * p.g;
+  const int start = p.starts[h * nbp1 + gb];
+  const int row_lo = (w - tp[gb]) * SEL_TILE_ROWS;
+  const int row_hi = min(rows, row_lo + SEL_TILE_ROWS);
+
+  const int tid = threadIdx.x;
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
+  for (int c = tid; c < BK * (D / 8); c += SEL_THREADS) {
+    const int row = c / (D / 8), col = c % (D / 8);
+    const int tok = tok0 + row;
+    vec8 x = zero8<T>();
+    if (tok < seq_end) x = load16<vec8>(kbase + (int64_t)tok * p.k_sn + col * 8);
+    store16(&Ks[row * KS + col * 8], x);
+  }
+  for (int c = tid; c < BK * (D / 8); c += SEL_THREADS) {
+    const int key = c % BK, dc = c / BK;
+    const int tok = tok0 + key;
+    vec8 x = zero8<T>();
+    if (tok < seq_end) x = load16<vec8>(vbase + (int64_t)tok * p.v_sn + dc * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) Vt[(dc * 8 + e) * VS + key] = x[e];
+  }
+  __syncthreads();
+
+  const int lane = tid & 63, wv = tid >> 6;
+  const int col = lane & 31, hh = lane >> 5;
+  const int32_t* toks = p.sel_tokens + (int64_t)h * p.cap + start;
+  const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)h * p.g * p.q_sh + hh * (D / 2);
+  const int64_t prow0 = ((int64_t)h * p.cap + start) * p.g;
+  T* opart = reinterpret_cast<T*>(p.o_part);
+
+  for (int sub = row_lo + wv * 32; sub < row_hi; sub += SEL_WG_ROWS) {
+    const int r = sub + col;
+    const bool valid = r < row_hi;
+    const int rr = valid ? r : row_hi - 1;
+    const int trank = rr / p.g;
+    const int head = rr - trank * p.g;
+    const int token = toks[trank];
+    const T* qrow = qbase + (int64_t)token * p.q_sn + (int64_t)head * p.q_sh;
+    vec8 qreg[NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) qreg[ks] = load16<vec8>(qrow + ks * 8);
+
+    f32x16 acc[NA];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        vec8 kf = load16<vec8>(&Ks[(a * 32 + col) * KS + hh * (D / 2) + ks * 8]);
+        acc[a] = Elem<T>::mfma32(kf, qreg[ks], acc[a]);
+      }
+    }
+    // causal mask: key index inside the block must be <= limit
+    const int limit = (token - seq_start) - b_local * BK;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+        float sv = key <= limit ? acc[a][i] : -INFINITY;
+        acc[a][i] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = fmaxf(mx, xor32(mx));
+    const float mref = (mx == -INFINITY) ? 0.f : mx * p.scale_log2;
+    float l = 0.f;
+    vec8 pk[NJ];
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pv = exp2f(acc[a][i] * p.scale_log2 - mref);
+        l += pv;
+        pk[a * 2 + (i >> 3)][i & 7] = (T)pv;
+      }
+    l += xor32(l);
+
+    f32x16 oacc[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        const T* vp = &Vt[(dt * 32 + col) * VS + 16 * j + 4 * hh];
+        vec4 lo = load8<vec4>(vp);
+        vec4 hi = load8<vec4>(vp + 8);
+        vec8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        oacc[dt] = Elem<T>::mfma32(vf, pk[j], oacc[dt]);
+      }
+    }
+    if (valid) {
+      const float inv_l = l > 0.f ? 1.f / l : 0.f;
+      const int64_t prow = prow0 + r;
+      T* orow = opart + prow * D + 4 * hh;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          vec4 x;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[e] = (T)(oacc[dt][4 * qd + e] * inv_l);
+          store8(orow + dt * 32 + 8 * qd, x);
+        }
+      if (hh == 0) p.lse_part[prow] = l > 0.f ? mref + log2f(l) : -INFINITY;
+    }
+  }
+}
+
+// Query-major merge.  D/8 lanes own one (query, head) row, 16 bytes each.
+template <typename T, int D>
+__global__ void __launch_bounds__(256)
+selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict__ lse_part,
+                          const int32_t* __restrict__ slot_of, int64_t cap, int64_t n_tokens, int hq,
+                          int g, int topk, T* __restrict__ o, int64_t o_sn, int64_t o_sh,
+                          float* __restrict__ lse) {
+  typedef typename Elem<T>::vec8 vec8;
+  constexpr int LPR = D / 8;
+  constexpr int RPB = 256 / LPR;
+  const int64_t R = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+  const int sub = threadIdx.x % LPR;
+  if (R >= n_tokens * hq) return;
+  const int64_t tok = R / hq;
+  const int hq_i = (int)(R - tok * hq);
+  const int kh = hq_i / g, head = hq_i - kh * g;
+  const int32_t* so = slot_of + ((int64_t)kh * n_tokens + tok) * topk;
+  const int64_t pbase = (int64_t)kh * cap;
+
+  // pass 1: LSE over the valid slots (lanes of the row split the slots)
+  float mx = -INFINITY;
+  for (int t = sub; t < topk; t += LPR) {
+    const int pidx = so[t];
+    if (pidx >= 0) mx = fmaxf(mx, lse_part[(pbase + pidx) * g + head]);
+  }
+#pragma unroll
+  for (int o_ = LPR / 2; o_ >= 1; o_ >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o_, LPR));
+  float sum = 0.f;
+  if (mx > -INFINITY) {
+    for (int t = sub; t < topk; t += LPR) {
+      const int pidx = so[t];
+      if (pidx >= 0) sum += exp2f(lse_part[(pbase + pidx) * g + head] - mx);
+    }
+  }
+#pragma unroll
+  for (int o_ = LPR / 2; o_ >= 1; o_ >>= 1) sum += __shfl_xor(sum, o_, LPR);
+  const float lse_tot = sum > 0.f ? mx + log2f(sum) : -INFINITY;
+
+  // pass 2: weighted sum of partial rows
+  float accv[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) accv[e] = 0.f;
+  if (sum > 0.f) {
+#pragma unroll 4
+    for (int t = 0; t < topk; ++t) {
+      const int pidx = so[t];
+      if (pidx < 0) continue;
+      const int64_t prow = (pbase + pidx) * g + head;
+      const float wgt = exp2f(lse_part[prow] - lse_tot);
+      vec8 x = load16<vec8>(o_part + prow * D + sub * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) accv[e] += wgt * (float)x[e];
+    }
+  }
+  vec8 out;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) out[e] = (T)accv[e];
+  store16(o + tok * o_sn + (int64_t)hq_i * o_sh + sub * 8, out);
+  if (sub == 0) lse[(int64_t)hq_i * n_tokens + tok] = lse_tot;
+}
+
+struct FwdWs {
+  size_t off_opart, off_lse, off_tiles, total;
+};
+
+static FwdWs fwd_ws_layout(int64_t n_tokens, int hq, int hkv, int d, int topk, int64_t max_blocks) {
+  FwdWs w;
+  const int g = hq / hkv;
+  const size_t cap = (size_t)n_tokens * topk;
+  w.off_opart = 0;
+  w.off_lse = align_up(cap * hkv * g * d * 2, 256);
+  w.off_tiles = w.off_lse + align_up(cap * hkv * g * 4, 256);
+  w.total = w.off_tiles + align_up((size_t)hkv * (max_blocks + 1) * 4, 256);
+  return w;
+}
+
+template <typename T, int D, int BK>
+static int launch_main(const SelFwdParams& p, int hkv, int64_t max_tiles, hipStream_t stream) {
+  constexpr int lds = SelLds<D, BK>::BYTES;
+  static bool attr_done = false;
+  if (!attr_done && lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)selattn_fwd_main_kernel<T, D, BK>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d B LDS): %s", lds, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_done = true;
+  }
+  dim3 grid((unsigned)max_tiles, hkv);
+  selattn_fwd_main_kernel<T, D, BK><<<grid, SEL_THREADS, lds, stream>>>(p);
+  return 0;
+}
+
+template <typename T>
+static int dispatch_main(int d, int bk, const SelFwdParams& p, int hkv, int64_t max_tiles,
+                         hipStream_t stream) {
+#define FSA_CASE(DD, BB) \
+  if (d == DD && bk == BB) return launch_main<T, DD, BB>(p, hkv, max_tiles, stream);
+  FSA_CASE(128, 64)
+  FSA_CASE(128, 32)
+  FSA_CASE(128, 128)
+  FSA_CASE(64, 32)
+  FSA_CASE(64, 64)
+  FSA_CASE(64, 128)
+  FSA_CASE(256, 32)
+  FSA_CASE(256, 64)
+  FSA_CASE(256, 128)
+#undef FSA_CASE
+  set_error("selected attention: head_dim=%d with block_size=%d is not supported "
+            "(head_dim in {64,128,256}, block_size in {32,64,128})", d, bk);
+  return FSA_ERR_UNSUPPORTED;
+}
+
+template <typename T>
+static int launch_reduce(int d, const void* o_part, const float* lse_part, const int32_t* slot_of,
+                         int64_t cap, int64_t n, int hq, int g, int topk, void* o, int64_t o_sn,
+                         int64_t o_sh, float* lse, hipStream_t stream) {
+  const int64_t rows = n * hq;
+#define FSA_CASE(DD)                                                                          \
+  if (d == DD) {                                                                              \
+    constexpr int RPB = 256 / (DD / 8);                                                       \
+    selattn_fwd_reduce_kernel<T, DD><<<(unsigned)((rows + RPB - 1) / RPB), 256, 0, stream>>>( \
+        (const T*)o_part, lse_part, slot_of, cap, n, hq, g, topk, (T*)o, o_sn, o_sh, lse);    \
+    return 0;                                                                                 \
+  }
+  FSA_CASE(64)
+  FSA_CASE(128)
+  FSA_CASE(256)
+#undef FSA_CASE
+  set_error("selected attention reduce: head_dim=%d not supported", d);
+  return FSA_ERR_UNSUPPORTED;
+}
+
+}  // namespace fsa
+
+using namespace fsa;
+
+extern "C" size_t fsa_selattn_fwd_workspace_bytes(int64_t total_tokens, int32_t num_q_heads,
+                                                  int32_t num_kv_heads, int32_t head_dim, int32_t topk,
+                                                  int64_t max_blocks) {
+  return fwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, max_blocks).total;
+}
+
+extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int32_t dtype,
+                               int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n,
+                               int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                               const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                               int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                               int32_t topk, int32_t block_size, int64_t max_blocks,
+                               float softmax_scale, const int32_t* cu_blocks, const int32_t* counts,
+                               const int32_t* starts, const int32_t* sel_tokens,
+                               const int32_t* slot_of, void* o, int64_t o_stride_n,
+                               int64_t o_stride_h, float* lse, void* workspace,
+                               size_t workspace_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FSA_CHECK_ARG(q && k && v && o && lse && cu_seqlens && cu_blocks && counts && starts && sel_tokens &&
+                    slot_of, "fsa_selattn_fwd: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_selattn_fwd: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
+                "fsa_selattn_fwd: num_q_heads must be a multiple of num_kv_heads");
+  FSA_CHECK_ARG(batch >= 1 && total_tokens >= 1 && topk >= 1, "fsa_selattn_fwd: empty problem");
+  FSA_CHECK_ARG(total_tokens * topk < ((int64_t)1 << 31), "fsa_selattn_fwd: total_tokens*topk >= 2^31");
+  FSA_CHECK_ARG((q_stride_n | q_stride_h | k_stride_n | k_stride_h | v_stride_n | v_stride_h |
+                 o_stride_n | o_stride_h) % 8 == 0,
+                "fsa_selattn_fwd: strides must be multiples of 8 elements (16-byte rows)");
+  const int g = num_q_heads / num_kv_heads;
+  FwdWs ws = fwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, max_blocks);
+  if (!workspace || workspace_bytes < ws.total) {
+    set_error("fsa_selattn_fwd: workspace too small (%zu < %zu)", workspace_bytes, ws.total);
+    return FSA_ERR_WORKSPACE;
+  }
+  char* wsp = (char*)workspace;
+  int32_t* tile_prefix = (int32_t*)(wsp + ws.off_tiles);
+  int rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, SEL_TILE_ROWS, tile_prefix, stream_);
+  if (rc) return rc;
+  const int64_t max_tiles = fsa_max_tiles(total_tokens, topk, g, SEL_TILE_ROWS, max_blocks);
+
+  SelFwdParams p;
+  p.q = q; p.k = k; p.v = v;
+  p.q_sn = q_stride_n; p.q_sh = q_stride_h;
+  p.k_sn = k_stride_n; p.k_sh = k_stride_h;
+  p.v_sn = v_stride_n; p.v_sh = v_stride_h;
+  p.cu_seqlens = cu_seqlens; p.cu_blocks = cu_blocks; p.counts = counts; p.starts = starts;
+  p.sel_tokens = sel_tokens; p.tile_prefix = tile_prefix;
+  p.batch = batch; p.max_blocks = max_blocks; p.cap = total_tokens * topk; p.g = g;
+  p.scale_log2 = softmax_scale * LOG2E;
+  p.o_part = wsp + ws.off_opart;
+  p.lse_part = (float*)(wsp + ws.off_lse);
+
+  rc = dtype == FSA_BF16
+           ? dispatch_main<__bf16>(head_dim, block_size, p, num_kv_heads, max_tiles, stream)
+           : dispatch_main<_Float16>(head_dim, block_size, p, num_kv_heads, max_tiles, stream);
+  if (rc) return rc;
+  FSA_CHECK_LAUNCH("fsa_selattn_fwd main");
+  rc = dtype == FSA_BF16
+           ? launch_reduce<__bf16>(head_dim, p.o_part, p.lse_part, slot_of, p.cap, total_tokens,
+                                   num_q_heads, g, topk, o, o_stride_n, o_stride_h, lse, stream)
+           : launch_reduce<_Float16>(head_dim, p.o_part, p.lse_part, slot_of, p.cap, total_tokens,
+                                     num_q_heads, g, topk, o, o_stride_n, o_stride_h, lse, stream);
+  if (rc) return rc;
+  FSA_CHECK_LAUNCH("fsa_selattn_fwd reduce");
+  return 0;
+}

@@ -1,0 +1,139 @@
+/*
+ * fsa_hip.h - C ABI of libfsa_gfx950.so: NSA selected attention (and the
+ * kernels around it) as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the name ends in _host;
+ *   - the library never allocates, frees or synchronises: outputs and
+ *     workspaces are passed in, kernels are enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL = the default stream);
+ *   - return value: 0 = ok, < 0 = invalid argument (see fsa_last_error()),
+ *     > 0 = a hipError_t from a launch;
+ *   - dtype codes: FSA_BF16 / FSA_FP16 for q, k, v, o and gradients;
+ *   - strides are in ELEMENTS; the innermost (head_dim) stride is 1;
+ *   - block ids inside topk_idx are local to the query's sequence, -1 = padding.
+ *
+ * The packed varlen layout is the reference's: q[N,Hq,D], k/v[N,Hkv,D],
+ * topk_idx[Hkv,N,T] int32, cu_seqlens[B+1] int32, lse[Hq,N] fp32 base 2
+ * (fsa/ops/FSA_topk_sparse_attention.py:1887-1932).
+ */
+#ifndef FSA_HIP_H
+#define FSA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FSA_BF16 0
+#define FSA_FP16 1
+
+#define FSA_ERR_INVALID (-1)
+#define FSA_ERR_UNSUPPORTED (-2)
+#define FSA_ERR_WORKSPACE (-3)
+
+/* Library version (major*10000 + minor*100 + patch). */
+int fsa_version(void);
+/* Human-readable description of the last error on the calling thread. */
+const char* fsa_last_error(void);
+
+/* ------------------------------------------------------------------------
+ * Inverted block->query index.
+ * Replaces: torch.bincount + build_block_to_token_triton + boolean compaction
+ * + cumsum/pad + index_mapping (fsa/ops/FSA_topk_sparse_attention.py:951-955,
+ * 59-135, 1016-1026, 621-668) and reorder_topk_idx
+ * (nsa_ref/ops/topk_sparse_attention.py:412-476), for all sequences and kv
+ * heads in one call.
+ *
+ * Global block id of block b of sequence s: cu_blocks[s] + b with
+ * cu_blocks = cumsum(ceil(len_s / block_size)).  max_blocks is any upper bound
+ * of cu_blocks[batch] known on the host, e.g. ceil(N / block_size) + batch.
+ *
+ *   cu_blocks  [batch+1]               out
+ *   counts     [Hkv, max_blocks]       out  entries per block
+ *   starts     [Hkv, max_blocks+1]     out  exclusive prefix of counts
+ *   sel_tokens [Hkv, N*T]              out  global query rows grouped by block,
+ *                                           ascending inside a block; -1 tail
+ *   slot_of    [Hkv, N, T]             out  position of (query, slot) in
+ *                                           sel_tokens, -1 for padding
+ * ---------------------------------------------------------------------- */
+size_t fsa_index_workspace_bytes(int64_t total_tokens, int32_t topk, int32_t num_kv_heads,
+                                 int64_t max_blocks);
+
+int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, int64_t topk_stride_n,
+                    const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                    int32_t num_kv_heads, int32_t topk, int32_t block_size, int64_t max_blocks,
+                    int32_t* cu_blocks, int32_t* counts, int32_t* starts, int32_t* sel_tokens,
+                    int32_t* slot_of, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Work list for the block-major kernels: tile_prefix[h, gb] = number of
+ * row tiles of blocks < gb, a row tile being `rows_per_tile` gathered
+ * (query, head-in-group) rows of one block.  tile_prefix is [Hkv, max_blocks+1].
+ * Replaces the rectangular grids with early exit of
+ * fsa/ops/FSA_topk_sparse_attention.py:758-821. */
+int fsa_build_tiles(const int32_t* counts, int32_t num_kv_heads, int64_t max_blocks,
+                    int32_t group_size, int32_t rows_per_tile, int32_t* tile_prefix, void* stream);
+
+/* Upper bound of the number of row tiles per kv head (host arithmetic only). */
+int64_t fsa_max_tiles(int64_t total_tokens, int32_t topk, int32_t group_size, int32_t rows_per_tile,
+                      int64_t max_blocks);
+
+/* ------------------------------------------------------------------------
+ * Selected attention forward.
+ * Replaces _topk_sparse_attention_fwd_opt (online_softmax/qk_kernel,
+ * qkv_kernel/forward_kernel_opt, reduce_output/reduce_kernel;
+ * fsa/ops/FSA_topk_sparse_attention.py:569-618, 671-907, 910-1116).
+ *
+ * Stage 1 (block-major): for every kv block, the queries that selected it are
+ * gathered into MFMA tiles; a normalised partial O row and its base-2 LSE are
+ * written per (query, block, head):
+ *     o_part   [Hkv, N*T, g, D]   same dtype as q
+ *     lse_part [Hkv, N*T, g]      fp32
+ * Stage 2 (query-major): the <= T partials of each (query, head) are merged.
+ * The workspace holds o_part, lse_part and the tile list.
+ * ---------------------------------------------------------------------- */
+size_t fsa_selattn_fwd_workspace_bytes(int64_t total_tokens, int32_t num_q_heads, int32_t num_kv_heads,
+                                       int32_t head_dim, int32_t topk, int64_t max_blocks);
+
+int fsa_selattn_fwd(const void* q, const void* k, const void* v, int32_t dtype,
+                    int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                    int64_t v_stride_n, int64_t v_stride_h,
+                    const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t topk,
+                    int32_t block_size, int64_t max_blocks, float softmax_scale,
+                    const int32_t* cu_blocks, const int32_t* counts, const int32_t* starts,
+                    const int32_t* sel_tokens, const int32_t* slot_of,
+                    void* o, int64_t o_stride_n, int64_t o_stride_h, float* lse /* [Hq, N] */,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Selected attention backward.
+ * Replaces _topk_sparse_attention_bwd_opt (backward_sum_o_do, backward_dkdv,
+ * dq_compute_kernel, dq_reduce_kernel; fsa/ops/FSA_topk_sparse_attention.py:
+ * 1715-1884, 1119-1321, 1547-1712; nsa_ref/ops/topk_sparse_attention.py:197-230).
+ * dq has q's layout, dk/dv have k's layout (already summed over the g heads
+ * of a group).  All outputs are fully overwritten.
+ * ---------------------------------------------------------------------- */
+size_t fsa_selattn_bwd_workspace_bytes(int64_t total_tokens, int32_t num_q_heads, int32_t num_kv_heads,
+                                       int32_t head_dim, int32_t topk, int32_t block_size,
+                                       int64_t max_blocks);
+
+int fsa_selattn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                    const float* lse, int32_t dtype,
+                    int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                    int64_t v_stride_n, int64_t v_stride_h, int64_t o_stride_n, int64_t o_stride_h,
+                    int64_t do_stride_n, int64_t do_stride_h,
+                    const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t topk,
+                    int32_t block_size, int64_t max_blocks, float softmax_scale,
+                    const int32_t* cu_blocks, const int32_t* counts, const int32_t* starts,
+                    const int32_t* sel_tokens, const int32_t* slot_of,
+                    void* dq, void* dk, void* dv /* contiguous [N,H,D] */,
+                    void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FSA_HIP_H */

@@ -1,0 +1,215 @@
+"""CPU oracle for NSA *selected attention* and its inverted index.
+
+TEST INFRASTRUCTURE ONLY - never imported by the product package.
+
+Restates, in plain PyTorch/numpy on the CPU, what the reference computes in
+  fsa/ops/FSA_topk_sparse_attention.py   (FSA kernels, index lists)
+  nsa_ref/ops/topk_sparse_attention.py   (per-query semantics)
+
+Pinning status (tests/test_oracle_selattn.py):
+  selected_attention_ref : pinned - dense-mask fp64 softmax, SDPA with an
+      explicit bool mask, closed forms (token 0, all-blocks == causal,
+      own-block only == block-diagonal causal), slot-permutation invariance.
+  selected_attention_grads_ref : pinned - autograd of the dense fp64
+      formulation and central finite differences on tiny inputs.
+  build_index_ref : pinned - brute-force Python loops, torch.bincount,
+      exclusive cumsum identity.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+LOG2E = 1.4426950408889634
+
+
+def _seq_bounds(cu_seqlens) -> list:
+    cu = [int(x) for x in cu_seqlens]
+    return [(cu[i], cu[i + 1]) for i in range(len(cu) - 1)]
+
+
+def selected_attention_ref(
+    q: torch.Tensor,  # [N, Hq, D]
+    k: torch.Tensor,  # [N, Hkv, D]
+    v: torch.Tensor,  # [N, Hkv, D]
+    topk_idx: torch.Tensor,  # [Hkv, N, T] int, -1 = padding, block ids local to the sequence
+    block_size: int,
+    cu_seqlens,
+    softmax_scale: Optional[float] = None,
+    q_chunk: int = 128,
+    dtype: torch.dtype = torch.float32,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """O[N,Hq,D] and base-2 LSE[Hq,N].
+
+    Per query i (sequence-local position) and q-head h with kv-head kh = h // g:
+    key set = { p : p // B_K in topk_idx[kh, i, :], p <= i, p < len }
+    (nsa_ref/ops/topk_sparse_attention.py:116-119,162;
+     fsa/ops/FSA_topk_sparse_attention.py:520),
+    s_p = scale * log2(e) * q.k  (FSA_topk_sparse_attention.py:318,523),
+    LSE2 = log2 sum 2^s_p  (FSA_topk_sparse_attention.py:256-261,273),
+    O = sum 2^(s_p - LSE2) v_p.
+    Differentiable (autograd) in q, k, v.
+    """
+    N, Hq, D = q.shape
+    Hkv = k.shape[1]
+    g = Hq // Hkv
+    T = topk_idx.shape[-1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    c = softmax_scale * LOG2E
+    qf, kf, vf = q.to(dtype), k.to(dtype), v.to(dtype)
+    o_chunks = []
+    lse_chunks = []
+    ar = torch.arange(block_size)
+    for (s0, s1) in _seq_bounds(cu_seqlens):
+        L = s1 - s0
+        ks, vs = kf[s0:s1], vf[s0:s1]
+        for i0 in range(0, L, q_chunk):
+            i1 = min(L, i0 + q_chunk)
+            C = i1 - i0
+            idx = topk_idx[:, s0 + i0 : s0 + i1, :].long()  # [Hkv, C, T]
+            kpos = idx[..., None] * block_size + ar  # [Hkv, C, T, B]
+            qpos = torch.arange(i0, i1)[None, :, None, None]
+            valid = (idx[..., None] >= 0) & (kpos <= qpos) & (kpos < L)
+            kpos = kpos.clamp(0, L - 1).reshape(Hkv, C, T * block_size)
+            valid = valid.reshape(Hkv, C, T * block_size)
+            hsel = torch.arange(Hkv)[:, None, None]
+            kg = ks[kpos, hsel]  # [Hkv, C, TB, D]
+            vg = vs[kpos, hsel]
+            qc = qf[s0 + i0 : s0 + i1].reshape(C, Hkv, g, D).permute(1, 0, 2, 3)  # [Hkv, C, g, D]
+            s = torch.einsum("hcgd,hckd->hcgk", qc, kg) * c
+            s = s.masked_fill(~valid[:, :, None, :], float("-inf"))
+            m = s.max(dim=-1, keepdim=True).values
+            m = torch.where(torch.isinf(m), torch.zeros_like(m), m)
+            p = torch.exp2(s - m)
+            l = p.sum(-1, keepdim=True)
+            lse = (m + torch.log2(l)).squeeze(-1)  # [Hkv, C, g]
+            o = torch.einsum("hcgk,hckd->hcgd", p / l, vg)
+            o_chunks.append(o.permute(1, 0, 2, 3).reshape(C, Hq, D))
+            lse_chunks.append(lse.permute(0, 2, 1).reshape(Hq, C))
+    return torch.cat(o_chunks, 0), torch.cat(lse_chunks, 1)
+
+
+def selected_attention_grads_ref(q, k, v, topk_idx, block_size, cu_seqlens, do, softmax_scale=None,
+                                 dtype=torch.float32, q_chunk: int = 128):
+    """(O, LSE2, dQ, dK, dV) through autograd of `selected_attention_ref`.
+
+    Mathematically the formulas of FSA_topk_sparse_attention.py:1229-1237 and
+    :1697-1709: dS = scale * P * (dP - delta), dQ = dS K, dK = sum over the
+    group's heads of dS^T Q, dV = sum over heads of P^T dO
+    (dK/dV head sum: FSA_topk_sparse_attention.py:1854-1855).
+    """
+    q_ = q.detach().to(dtype).requires_grad_(True)
+    k_ = k.detach().to(dtype).requires_grad_(True)
+    v_ = v.detach().to(dtype).requires_grad_(True)
+    o, lse = selected_attention_ref(q_, k_, v_, topk_idx, block_size, cu_seqlens, softmax_scale,
+                                    q_chunk=q_chunk, dtype=dtype)
+    (o * do.to(dtype)).sum().backward()
+    return o.detach(), lse.detach(), q_.grad, k_.grad, v_.grad
+
+
+def dense_mask(topk_idx: torch.Tensor, block_size: int, cu_seqlens) -> torch.Tensor:
+    """Bool [Hkv, N, N]: mask[kh, i, p] = key p (global row) visible to query i."""
+    Hkv, N, T = topk_idx.shape
+    mask = torch.zeros(Hkv, N, N, dtype=torch.bool)
+    for (s0, s1) in _seq_bounds(cu_seqlens):
+        L = s1 - s0
+        pos = torch.arange(L)
+        blk = pos // block_size
+        for kh in range(Hkv):
+            idx = topk_idx[kh, s0:s1].long()  # [L, T]
+            sel = (idx[:, :, None] == blk[None, None, :]).any(1)  # [L(query), L(key)]
+            sel &= pos[None, :] <= pos[:, None]
+            mask[kh, s0:s1, s0:s1] = sel
+    return mask
+
+
+def selected_attention_dense_ref(q, k, v, topk_idx, block_size, cu_seqlens, softmax_scale=None,
+                                 dtype=torch.float64):
+    """Same quantity via an explicit [N, N] mask and torch.softmax (small N only)."""
+    N, Hq, D = q.shape
+    Hkv = k.shape[1]
+    g = Hq // Hkv
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    mask = dense_mask(topk_idx, block_size, cu_seqlens)  # [Hkv, N, N]
+    qf, kf, vf = q.to(dtype), k.to(dtype), v.to(dtype)
+    kx = kf.repeat_interleave(g, dim=1)
+    vx = vf.repeat_interleave(g, dim=1)
+    mx = mask.repeat_interleave(g, dim=0)  # [Hq, N, N]
+    s = torch.einsum("ihd,phd->hip", qf, kx) * softmax_scale
+    s = s.masked_fill(~mx, float("-inf"))
+    p = torch.softmax(s, dim=-1)
+    o = torch.einsum("hip,phd->ihd", p, vx)
+    lse2 = torch.logsumexp(s, dim=-1) * LOG2E
+    return o, lse2
+
+
+def build_index_ref(topk_idx: torch.Tensor, cu_seqlens, block_size: int):
+    """Inverted block->query index, all sequences at once, global numbering.
+
+    Block b of sequence s has global id cu_blocks[s] + b with
+    cu_blocks = cumsum(ceil(len_s / B_K)).  Per kv head:
+      counts[gb]      = number of (query, slot) entries naming that block
+                        (torch.bincount, FSA_topk_sparse_attention.py:951-955)
+      starts          = exclusive cumsum of counts (:1018), length NB + 1
+      sel_tokens[p]   = query ids (global rows) grouped by block, ascending
+                        inside a block (row-major compaction of a
+                        [nblk, N] table, :1016)
+      slot_of[i, t]   = position p of entry (i, t) in sel_tokens, -1 for
+                        padding; slot_of - starts[gb] is the reference's
+                        token_index_mapping (:641-649)
+    Entries that are negative or name a block past the sequence end are
+    ignored.  Returns numpy int32 arrays (cu_blocks, counts, starts,
+    sel_tokens[Hkv, N*T] (-1 tail), slot_of[Hkv, N, T]).
+    """
+    t = topk_idx.cpu().numpy().astype(np.int64)
+    Hkv, N, T = t.shape
+    bounds = _seq_bounds(cu_seqlens)
+    nblk = [(s1 - s0 + block_size - 1) // block_size for (s0, s1) in bounds]
+    cu_blocks = np.zeros(len(bounds) + 1, dtype=np.int64)
+    cu_blocks[1:] = np.cumsum(nblk)
+    NB = int(cu_blocks[-1])
+    gkey = np.full((Hkv, N, T), NB, dtype=np.int64)
+    for s, (s0, s1) in enumerate(bounds):
+        loc = t[:, s0:s1, :]
+        ok = (loc >= 0) & (loc < nblk[s])
+        gkey[:, s0:s1, :] = np.where(ok, loc + cu_blocks[s], NB)
+    counts = np.zeros((Hkv, NB), dtype=np.int32)
+    starts = np.zeros((Hkv, NB + 1), dtype=np.int32)
+    sel_tokens = np.full((Hkv, N * T), -1, dtype=np.int32)
+    slot_of = np.full((Hkv, N, T), -1, dtype=np.int32)
+    for h in range(Hkv):
+        flat = gkey[h].reshape(-1)
+        order = np.argsort(flat, kind="stable")
+        skeys = flat[order]
+        nvalid = int((skeys < NB).sum())
+        counts[h] = np.bincount(skeys[:nvalid], minlength=NB)[:NB]
+        starts[h, 1:] = np.cumsum(counts[h])
+        sel_tokens[h, :nvalid] = (order[:nvalid] // T).astype(np.int32)
+        so = slot_of[h].reshape(-1)
+        so[order[:nvalid]] = np.arange(nvalid, dtype=np.int32)
+    return cu_blocks.astype(np.int32), counts, starts, sel_tokens, slot_of
+
+
+def count_pairs(topk_idx: torch.Tensor, block_size: int, cu_seqlens) -> Tuple[int, int]:
+    """(valid (query, block) pairs summed over kv heads,
+        unmasked (query, key) pairs summed over kv heads)."""
+    Hkv, N, T = topk_idx.shape
+    pairs = 0
+    keys = 0
+    for (s0, s1) in _seq_bounds(cu_seqlens):
+        L = s1 - s0
+        idx = topk_idx[:, s0:s1].long()
+        pos = torch.arange(L)[None, :, None]
+        nb = (L + block_size - 1) // block_size
+        ok = (idx >= 0) & (idx < nb)
+        lo = idx * block_size
+        n = (torch.minimum(pos, lo + block_size - 1) - lo + 1).clamp(min=0)
+        n = torch.where(ok, n, torch.zeros_like(n))
+        pairs += int(ok.sum())
+        keys += int(n.sum())
+    return pairs, keys

@@ -1,0 +1,69 @@
+"""GPU parity: HIP selected-attention forward and index vs the CPU oracle.
+
+Tolerances (from the task statement): O max-abs 2e-2 for bf16, 5e-3 for fp16;
+base-2 LSE max-abs 1e-3; index lists bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from fsa_hip import ops
+from fsa_hip.synth import make_qkv, make_topk_idx
+from oracle import selattn as orc
+
+pytestmark = pytest.mark.gpu
+
+O_TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
+LSE_TOL = 1e-3
+
+
+def _run_case(dev, cu, hq, hkv, d, bk, t, dtype, seed, std=1.0):
+    n = cu[-1]
+    q, k, v = make_qkv(n, hq, hkv, d, dtype, seed=seed, std=std, with_do=False)
+    topk = make_topk_idx(cu, hkv, bk, t, seed=seed + 1)
+    cu_t = torch.tensor(cu, dtype=torch.int32)
+    index = ops.build_index(topk.to(dev), cu_t.to(dev), bk)
+    o, lse = ops.selattn_fwd(q.to(dev), k.to(dev), v.to(dev), index)
+    torch.cuda.synchronize()
+    o_ref, lse_ref = orc.selected_attention_ref(q.float(), k.float(), v.float(), topk, bk, cu)
+    return index, topk, o.float().cpu(), lse.cpu(), o_ref, lse_ref
+
+
+def _check_index(index, topk, cu, bk):
+    cu_blocks, counts, starts, sel_tokens, slot_of = orc.build_index_ref(topk, cu, bk)
+    nb = int(cu_blocks[-1])
+    assert np.array_equal(index.cu_blocks.cpu().numpy(), cu_blocks)
+    got_counts = index.counts.cpu().numpy()
+    assert np.array_equal(got_counts[:, :nb], counts)
+    assert (got_counts[:, nb:] == 0).all()
+    got_starts = index.starts.cpu().numpy()
+    assert np.array_equal(got_starts[:, : nb + 1], starts)
+    assert np.array_equal(index.sel_tokens.cpu().numpy(), sel_tokens)
+    assert np.array_equal(index.slot_of.cpu().numpy(), slot_of)
+
+
+CASES = [
+    # cu_seqlens, Hq, Hkv, D, B_K, T, dtype
+    ([0, 1024], 4, 4, 128, 64, 16, torch.bfloat16),
+    ([0, 2048], 8, 4, 128, 64, 16, torch.bfloat16),
+    ([0, 1536], 16, 4, 128, 64, 16, torch.bfloat16),
+    ([0, 700, 701, 1900, 2048], 8, 2, 128, 64, 8, torch.bfloat16),   # ragged varlen, 1-token seq
+    ([0, 1000], 6, 2, 128, 32, 4, torch.float16),                    # g = 3, partial last block
+    ([0, 2048], 4, 2, 256, 128, 8, torch.float16),
+    ([0, 512], 4, 1, 64, 64, 16, torch.bfloat16),                    # T > number of blocks
+    ([0, 33], 2, 2, 128, 64, 16, torch.bfloat16),                    # shorter than one block
+]
+
+
+@pytest.mark.parametrize("cu,hq,hkv,d,bk,t,dtype", CASES)
+def test_fwd_matches_oracle(dev, cu, hq, hkv, d, bk, t, dtype):
+    print(f"case cu={cu} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    std = 0.5 if d == 256 else 1.0
+    index, topk, o, lse, o_ref, lse_ref = _run_case(dev, cu, hq, hkv, d, bk, t, dtype, seed=42, std=std)
+    _check_index(index, topk, cu, bk)
+    assert torch.isfinite(o).all() and torch.isfinite(lse).all()
+    err_o = (o - o_ref).abs().max().item()
+    err_l = (lse - lse_ref).abs().max().item()
+    print(f"  max|dO|={err_o:.3e} max|dLSE|={err_l:.3e}", flush=True)
+    assert err_o <= O_TOL[dtype]
+    assert err_l <= LSE_TOL
