@@ -97,24 +97,22 @@ radix_hist_kernel(const uint32_t* __restrict__ keys, int64_t n_items, int shift,
   table[((int64_t)h * 256 + tid) * ntiles + tile] = hist[tid];
 }
 
-// in-place exclusive scan of table[h][0 .. 256*ntiles)
-__global__ void __launch_bounds__(SCAN_THREADS)
-radix_scan_kernel(uint32_t* __restrict__ table, int ntiles) {
-  const int h = blockIdx.x;
-  const int64_t m = (int64_t)256 * ntiles;
-  uint32_t* t = table + (int64_t)h * m;
-  const int64_t per = (m + SCAN_THREADS - 1) / SCAN_THREADS;
-  const int64_t lo = (int64_t)threadIdx.x * per;
-  const int64_t hi = lo + per < m ? lo + per : m;
-  int sum = 0;
-  for (int64_t i = lo; i < hi; ++i) sum += (int)t[i];
-  int total;
-  int run = block_exclusive_scan(sum, &total);
-  for (int64_t i = lo; i < hi; ++i) {
-    int c = (int)t[i];
-    t[i] = (uint32_t)run;
-    run += c;
+// Per (head, digit) row: in-place exclusive scan over the tiles; the row total
+// goes to totals[h][digit] (the scatter kernel scans those 256 values itself).
+__global__ void __launch_bounds__(256)
+radix_scan_kernel(uint32_t* __restrict__ table, int ntiles, uint32_t* __restrict__ totals) {
+  const int d = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  uint32_t* row = table + ((int64_t)h * 256 + d) * ntiles;
+  int carry = 0;
+  for (int base = 0; base < ntiles; base += 256) {
+    const int i = base + tid;
+    const int v = i < ntiles ? (int)row[i] : 0;
+    int total;
+    const int ex = block_exclusive_scan(v, &total);
+    if (i < ntiles) row[i] = (uint32_t)(carry + ex);
+    carry += total;
   }
+  if (tid == 0) totals[h * 256 + d] = (uint32_t)carry;
 }
 
 // Stable scatter of one 8-bit digit.  Item order inside a tile is
@@ -122,7 +120,8 @@ radix_scan_kernel(uint32_t* __restrict__ table, int ntiles) {
 __global__ void __launch_bounds__(RS_THREADS)
 radix_scatter_kernel(const uint32_t* __restrict__ keys_in, const uint32_t* __restrict__ vals_in,
                      uint32_t* __restrict__ keys_out, uint32_t* __restrict__ vals_out,
-                     int64_t n_items, int shift, int ntiles, const uint32_t* __restrict__ table) {
+                     int64_t n_items, int shift, int ntiles, const uint32_t* __restrict__ table,
+                     const uint32_t* __restrict__ totals) {
   __shared__ uint32_t cnt[RS_WAVES][256];
   const int h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
   const int lane = tid & (WAVE - 1), w = tid / WAVE;
@@ -158,9 +157,11 @@ radix_scatter_kernel(const uint32_t* __restrict__ keys_in, const uint32_t* __res
     __builtin_amdgcn_wave_barrier();
   }
   __syncthreads();
+  int all_items;
+  const int digit_base = block_exclusive_scan((int)totals[h * 256 + tid], &all_items);
   {  // per digit: global base of this tile + exclusive prefix over waves
     const int d = tid;
-    uint32_t run = table[((int64_t)h * 256 + d) * ntiles + tile];
+    uint32_t run = (uint32_t)digit_base + table[((int64_t)h * 256 + d) * ntiles + tile];
 #pragma unroll
     for (int ww = 0; ww < RS_WAVES; ++ww) {
       uint32_t c = cnt[ww][d];
@@ -246,7 +247,7 @@ tiles_kernel(const int32_t* __restrict__ counts, int64_t max_blocks, int group_s
 using namespace fsa;
 
 static void index_ws_layout(int64_t n_items, int hkv, size_t* off_keys, size_t* off_vals,
-                            size_t* off_table, size_t* total) {
+                            size_t* off_table, size_t* off_totals, size_t* total) {
   const size_t buf = align_up((size_t)n_items * hkv * 4, 256);
   const int64_t ntiles = (n_items + RS_TILE - 1) / RS_TILE;
   off_keys[0] = 0;
@@ -254,14 +255,15 @@ static void index_ws_layout(int64_t n_items, int hkv, size_t* off_keys, size_t* 
   off_vals[0] = 2 * buf;
   off_vals[1] = 3 * buf;
   *off_table = 4 * buf;
-  *total = 4 * buf + align_up((size_t)hkv * 256 * ntiles * 4, 256);
+  *off_totals = *off_table + align_up((size_t)hkv * 256 * ntiles * 4, 256);
+  *total = *off_totals + align_up((size_t)hkv * 256 * 4, 256);
 }
 
 extern "C" size_t fsa_index_workspace_bytes(int64_t total_tokens, int32_t topk, int32_t num_kv_heads,
                                             int64_t max_blocks) {
   (void)max_blocks;
-  size_t ok[2], ov[2], ot, total;
-  index_ws_layout(total_tokens * topk, num_kv_heads, ok, ov, &ot, &total);
+  size_t ok[2], ov[2], ot, ott, total;
+  index_ws_layout(total_tokens * topk, num_kv_heads, ok, ov, &ot, &ott, &total);
   return total;
 }
 
@@ -281,8 +283,8 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
                 "fsa_build_index: max_blocks=%lld out of range", (long long)max_blocks);
   const int64_t n_items = total_tokens * topk;
   FSA_CHECK_ARG(n_items < ((int64_t)1 << 31), "fsa_build_index: total_tokens*topk must be < 2^31");
-  size_t ok[2], ov[2], ot, total;
-  index_ws_layout(n_items, num_kv_heads, ok, ov, &ot, &total);
+  size_t ok[2], ov[2], ot, ott, total;
+  index_ws_layout(n_items, num_kv_heads, ok, ov, &ot, &ott, &total);
   if (workspace == nullptr || workspace_bytes < total) {
     set_error("fsa_build_index: workspace too small (%zu < %zu)", workspace_bytes, total);
     return FSA_ERR_WORKSPACE;
@@ -291,6 +293,7 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
   uint32_t* keys[2] = {(uint32_t*)(ws + ok[0]), (uint32_t*)(ws + ok[1])};
   uint32_t* vals[2] = {(uint32_t*)(ws + ov[0]), (uint32_t*)(ws + ov[1])};
   uint32_t* table = (uint32_t*)(ws + ot);
+  uint32_t* totals = (uint32_t*)(ws + ott);
   const int ntiles = (int)((n_items + RS_TILE - 1) / RS_TILE);
   const uint32_t sentinel = (uint32_t)max_blocks;
 
@@ -306,10 +309,10 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
   for (int p = 0; p < passes; ++p) {
     dim3 g_tiles(ntiles, num_kv_heads);
     radix_hist_kernel<<<g_tiles, RS_THREADS, 0, stream>>>(keys[cur], n_items, 8 * p, ntiles, table);
-    radix_scan_kernel<<<num_kv_heads, SCAN_THREADS, 0, stream>>>(table, ntiles);
+    radix_scan_kernel<<<dim3(256, num_kv_heads), 256, 0, stream>>>(table, ntiles, totals);
     radix_scatter_kernel<<<g_tiles, RS_THREADS, 0, stream>>>(keys[cur], vals[cur], keys[cur ^ 1],
                                                              vals[cur ^ 1], n_items, 8 * p, ntiles,
-                                                             table);
+                                                             table, totals);
     cur ^= 1;
   }
   finalize_items_kernel<<<g_items, 256, 0, stream>>>(keys[cur], vals[cur], n_items, topk, sentinel,

@@ -39,16 +39,17 @@ struct SelFwdParams {
 
 constexpr int SEL_THREADS = 256;
 constexpr int SEL_WG_ROWS = 128;                 // rows per pass of the 4 waves
-constexpr int SEL_TILE_ROWS = 4 * SEL_WG_ROWS;   // rows per work-group
+constexpr int SEL_TILE_ROWS = 8 * SEL_WG_ROWS;   // rows per work-group
 
 template <int D, int BK> struct SelLds {
   static constexpr int KS = D + 8;   // K row stride in elements (16 B pad: bank spread)
   static constexpr int VS = BK + 4;  // V^T row stride in elements
   static constexpr int BYTES = (BK * KS + D * VS) * 2;
+  static constexpr int MIN_WAVES = (D <= 128 && BK <= 64) ? 2 : 1;  // waves per SIMD the register budget allows
 };
 
 template <typename T, int D, int BK>
-__global__ void __launch_bounds__(SEL_THREADS)
+__global__ void __launch_bounds__(SEL_THREADS, (SelLds<D, BK>::MIN_WAVES))
 selattn_fwd_main_kernel(SelFwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
@@ -103,17 +104,41 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   const int64_t prow0 = ((int64_t)h * p.cap + start) * p.g;
   T* opart = reinterpret_cast<T*>(p.o_part);
 
-  for (int sub = row_lo + wv * 32; sub < row_hi; sub += SEL_WG_ROWS) {
+  // Software pipeline over the wave's 32-row sub-tiles: token ids are fetched
+  // two steps ahead, Q rows one step ahead of the MFMA work.
+  auto row_token = [&](int sub_, int& head_) {
+    const int r_ = min(sub_ + col, row_hi - 1);
+    const int trank_ = r_ / p.g;
+    head_ = r_ - trank_ * p.g;
+    return toks[trank_];
+  };
+  int sub = row_lo + wv * 32;
+  if (sub >= row_hi) return;
+  int head_n, head_nn = 0;
+  int tok_n = row_token(sub, head_n);
+  vec8 qnext[NKS];
+  {
+    const T* qrow = qbase + (int64_t)tok_n * p.q_sn + (int64_t)head_n * p.q_sh;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) qnext[ks] = load16<vec8>(qrow + ks * 8);
+  }
+  int tok_nn = (sub + SEL_WG_ROWS < row_hi) ? row_token(sub + SEL_WG_ROWS, head_nn) : 0;
+
+  for (; sub < row_hi; sub += SEL_WG_ROWS) {
     const int r = sub + col;
     const bool valid = r < row_hi;
-    const int rr = valid ? r : row_hi - 1;
-    const int trank = rr / p.g;
-    const int head = rr - trank * p.g;
-    const int token = toks[trank];
-    const T* qrow = qbase + (int64_t)token * p.q_sn + (int64_t)head * p.q_sh;
+    const int token = tok_n;
     vec8 qreg[NKS];
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qreg[ks] = load16<vec8>(qrow + ks * 8);
+    for (int ks = 0; ks < NKS; ++ks) qreg[ks] = qnext[ks];
+    tok_n = tok_nn;
+    head_n = head_nn;
+    if (sub + SEL_WG_ROWS < row_hi) {
+      const T* qrow = qbase + (int64_t)tok_n * p.q_sn + (int64_t)head_n * p.q_sh;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) qnext[ks] = load16<vec8>(qrow + ks * 8);
+    }
+    if (sub + 2 * SEL_WG_ROWS < row_hi) tok_nn = row_token(sub + 2 * SEL_WG_ROWS, head_nn);
 
     f32x16 acc[NA];
 #pragma unroll
@@ -151,36 +176,37 @@ selattn_fwd_main_kernel(SelFwdParams p) {
         pk[a * 2 + (i >> 3)][i & 7] = (T)pv;
       }
     l += xor32(l);
-
-    f32x16 oacc[NDT];
+    const float inv_l = l > 0.f ? 1.f / l : 0.f;
+    const int64_t prow = prow0 + r;
+    // Partial rows are stored in the lane-native order
+    //   pos = hh*(D/2) + dt*16 + i   <->   d = dt*32 + 8*(i/4) + 4*hh + i%4
+    // so that every lane owns one contiguous half row (16-byte stores); the
+    // merge kernel undoes the permutation when it writes O.
+    T* orow = opart + prow * D + hh * (D / 2);
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
+      f32x16 oacc;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+      for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         const T* vp = &Vt[(dt * 32 + col) * VS + 16 * j + 4 * hh];
         vec4 lo = load8<vec4>(vp);
         vec4 hi = load8<vec4>(vp + 8);
         vec8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        oacc[dt] = Elem<T>::mfma32(vf, pk[j], oacc[dt]);
+        oacc = Elem<T>::mfma32(vf, pk[j], oacc);
+      }
+      if (valid) {
+#pragma unroll
+        for (int c8 = 0; c8 < 2; ++c8) {
+          vec8 x;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) x[e] = (T)(oacc[c8 * 8 + e] * inv_l);
+          store16(orow + dt * 16 + c8 * 8, x);
+        }
       }
     }
-    if (valid) {
-      const float inv_l = l > 0.f ? 1.f / l : 0.f;
-      const int64_t prow = prow0 + r;
-      T* orow = opart + prow * D + 4 * hh;
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          vec4 x;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) x[e] = (T)(oacc[dt][4 * qd + e] * inv_l);
-          store8(orow + dt * 32 + 8 * qd, x);
-        }
-      if (hh == 0) p.lse_part[prow] = l > 0.f ? mref + log2f(l) : -INFINITY;
-    }
+    if (valid && hh == 0) p.lse_part[prow] = l > 0.f ? mref + log2f(l) : -INFINITY;
   }
 }
 
@@ -238,10 +264,22 @@ selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict_
       for (int e = 0; e < 8; ++e) accv[e] += wgt * (float)x[e];
     }
   }
-  vec8 out;
+  // un-permute: positions [8*sub, 8*sub+8) of a partial row are two runs of 4 dims
+  {
+    typedef typename Elem<T>::vec4 vec4;
+    const int pos = sub * 8;
+    const int hh = pos / (D / 2), rem = pos % (D / 2);
+    const int dt = rem / 16, i0 = rem % 16;  // i0 in {0, 8}
+    T* orow = o + tok * o_sn + (int64_t)hq_i * o_sh + dt * 32 + 4 * hh + 8 * (i0 >> 2);
+    vec4 a, b;
 #pragma unroll
-  for (int e = 0; e < 8; ++e) out[e] = (T)accv[e];
-  store16(o + tok * o_sn + (int64_t)hq_i * o_sh + sub * 8, out);
+    for (int e = 0; e < 4; ++e) {
+      a[e] = (T)accv[e];
+      b[e] = (T)accv[4 + e];
+    }
+    store8(orow, a);
+    store8(orow + 8, b);
+  }
   if (sub == 0) lse[(int64_t)hq_i * n_tokens + tok] = lse_tot;
 }
 
