@@ -67,6 +67,28 @@ template <typename T> __device__ __forceinline__ typename Elem<T>::vec8 zero8() 
   return __builtin_bit_cast(typename Elem<T>::vec8, z);
 }
 
+// LDS transposing read (gfx950 ds_read_b64_tr_b16).  Inside every group of 16
+// lanes, lane j receives, for e = 0..3, element (j % 4) of the 8-byte word whose
+// address was supplied by lane 4*e + j/4 of the group.  With lane s pointing at
+// M[r0 + (s%16)/4][c0 + 4*(s%4) ..], lane j therefore gets M[r0 + e][c0 + j],
+// e = 0..3: four consecutive rows of one column out of a row-major tile.
+template <typename T> __device__ __forceinline__ typename Elem<T>::vec4 lds_read_tr4(const T* p) {
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) s16x4* lds_ptr;
+  s16x4 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+  return __builtin_bit_cast(typename Elem<T>::vec4, r);
+}
+
+// Eight values of one column (two runs of four consecutive rows, 8 rows apart)
+// of a row-major LDS tile, as the k-contiguous MFMA operand of a contraction
+// over the tile's rows.  `p` is this lane's address for row r0 + (lane%16)/4.
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::vec8 lds_read_tr8(const T* p, int stride8rows) {
+  typename Elem<T>::vec4 lo = lds_read_tr4<T>(p);
+  typename Elem<T>::vec4 hi = lds_read_tr4<T>(p + stride8rows);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
 // largest i in [0, n) with a[i] <= x, for ascending a[0..n) with a[0] <= x

@@ -43,8 +43,8 @@ constexpr int SEL_TILE_ROWS = 8 * SEL_WG_ROWS;   // rows per work-group
 
 template <int D, int BK> struct SelLds {
   static constexpr int KS = D + 8;   // K row stride in elements (16 B pad: bank spread)
-  static constexpr int VS = BK + 4;  // V^T row stride in elements
-  static constexpr int BYTES = (BK * KS + D * VS) * 2;
+  static constexpr int VS = D + 16;  // V row stride in elements (32 B pad for the transposing reads)
+  static constexpr int BYTES = (BK * KS + BK * VS) * 2;
   static constexpr int MIN_WAVES = (D <= 128 && BK <= 64) ? 2 : 1;  // waves per SIMD the register budget allows
 };
 
@@ -52,7 +52,6 @@ template <typename T, int D, int BK>
 __global__ void __launch_bounds__(SEL_THREADS, (SelLds<D, BK>::MIN_WAVES))
 selattn_fwd_main_kernel(SelFwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
-  typedef typename Elem<T>::vec4 vec4;
   constexpr int KS = SelLds<D, BK>::KS, VS = SelLds<D, BK>::VS;
   constexpr int NA = BK / 32;   // S^T accumulators (32 keys each)
   constexpr int NKS = D / 16;   // k-steps of QK^T
@@ -60,7 +59,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   constexpr int NJ = BK / 16;   // k-steps of PV
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* Ks = reinterpret_cast<T*>(smem);
-  T* Vt = Ks + BK * KS;
+  T* Vs = Ks + BK * KS;
 
   const int h = blockIdx.y;
   const int64_t nbp1 = p.max_blocks + 1;
@@ -88,12 +87,11 @@ selattn_fwd_main_kernel(SelFwdParams p) {
     store16(&Ks[row * KS + col * 8], x);
   }
   for (int c = tid; c < BK * (D / 8); c += SEL_THREADS) {
-    const int key = c % BK, dc = c / BK;
-    const int tok = tok0 + key;
+    const int row = c / (D / 8), col = c % (D / 8);
+    const int tok = tok0 + row;
     vec8 x = zero8<T>();
-    if (tok < seq_end) x = load16<vec8>(vbase + (int64_t)tok * p.v_sn + dc * 8);
-#pragma unroll
-    for (int e = 0; e < 8; ++e) Vt[(dc * 8 + e) * VS + key] = x[e];
+    if (tok < seq_end) x = load16<vec8>(vbase + (int64_t)tok * p.v_sn + col * 8);
+    store16(&Vs[row * VS + col * 8], x);
   }
   __syncthreads();
 
@@ -103,6 +101,9 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)h * p.g * p.q_sh + hh * (D / 2);
   const int64_t prow0 = ((int64_t)h * p.cap + start) * p.g;
   T* opart = reinterpret_cast<T*>(p.o_part);
+  // this lane's address inside V for the transposing reads of O^T = V^T P^T:
+  // keys 4*hh + (lane%16)/4 (+ 16*j, + 8), dims 16*((lane/16)&1) + 4*(lane%4) (+ 32*dt)
+  const T* vtr = Vs + (4 * hh + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   // Software pipeline over the wave's 32-row sub-tiles: token ids are fetched
   // two steps ahead, Q rows one step ahead of the MFMA work.
@@ -190,10 +191,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const T* vp = &Vt[(dt * 32 + col) * VS + 16 * j + 4 * hh];
-        vec4 lo = load8<vec4>(vp);
-        vec4 hi = load8<vec4>(vp + 8);
-        vec8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        vec8 vf = lds_read_tr8<T>(vtr + 16 * j * VS + dt * 32, 8 * VS);
         oacc = Elem<T>::mfma32(vf, pk[j], oacc);
       }
       if (valid) {

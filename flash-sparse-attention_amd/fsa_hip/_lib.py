@@ -29,6 +29,12 @@ SIGNATURES = {
                                   vp, i32, i64, i32, i32, i32, i32, i32, i64, f32,
                                   vp, vp, vp, vp, vp,
                                   vp, i64, i64, vp, vp, sz, vp]),
+    "fsa_selattn_bwd_workspace_bytes": (sz, [i64, i32, i32, i32, i32, i32, i64]),
+    "fsa_selattn_bwd": (C.c_int, [vp, vp, vp, vp, vp, vp, i32,
+                                  i64, i64, i64, i64, i64, i64, i64, i64, i64, i64,
+                                  vp, i32, i64, i32, i32, i32, i32, i32, i64, f32,
+                                  vp, vp, vp, vp, vp,
+                                  vp, vp, vp, vp, sz, vp]),
 }
 
 

@@ -108,3 +108,39 @@ def selattn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, index: SelInd
         _ptr(o), o.stride(0), o.stride(1), _ptr(lse), _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_selattn_fwd")
     return o, lse
+
+
+def selattn_bwd(q, k, v, o, do, lse, index: SelIndex, softmax_scale: Optional[float] = None):
+    """Selected attention backward: returns (dq, dk, dv) in the input dtype."""
+    _check_qkv(q, k, v)
+    _require_cuda(o, do, lse)
+    assert o.dtype == q.dtype and do.dtype == q.dtype and lse.dtype == torch.float32
+    assert o.shape == q.shape and do.shape == q.shape
+    lib = _lib.load()
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if do.stride(2) != 1:
+        do = do.contiguous()
+    if o.stride(2) != 1:
+        o = o.contiguous()
+    lse = lse.contiguous()
+    dev = q.device
+    dq = torch.empty((n, hq, d), dtype=q.dtype, device=dev)
+    dk = torch.empty((n, hkv, d), dtype=q.dtype, device=dev)
+    dv = torch.empty((n, hkv, d), dtype=q.dtype, device=dev)
+    ws_bytes = lib.fsa_selattn_bwd_workspace_bytes(n, hq, hkv, d, index.topk, index.block_size,
+                                                   index.max_blocks)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    rc = lib.fsa_selattn_bwd(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _DTYPE[q.dtype],
+        q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+        o.stride(0), o.stride(1), do.stride(0), do.stride(1),
+        _ptr(index.cu_seqlens), index.batch, n, hq, hkv, d, index.topk, index.block_size,
+        index.max_blocks, float(softmax_scale),
+        _ptr(index.cu_blocks), _ptr(index.counts), _ptr(index.starts), _ptr(index.sel_tokens),
+        _ptr(index.slot_of),
+        _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws_bytes, _stream(dev))
+    _lib.check(rc, "fsa_selattn_bwd")
+    return dq, dk, dv
