@@ -1,0 +1,218 @@
+#!/usr/bin/env python3
+"""Benchmark of the selected-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" = index build + forward + backward of NSA selected attention for the
+three GQA groups of the headline configuration (single varlen sequence of 65536
+tokens, 4 kv heads, Hq = 4 / 8 / 16, head_dim 128, block 64, top-16, bf16,
+synthetic N(0,1) inputs and the seeded synthetic block lists).  Inputs are
+resident in HBM before the timed region.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "flash-sparse-attention_amd"))
+
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+
+METRIC = "selected-attn fwd+bwd ms & TFLOP/s at 64K, B_K=64, T=16, GQA 1-4; roofline %"
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seq-len", type=int, default=65536)
+    ap.add_argument("--groups", type=str, default="1,2,4")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seq-len", type=int, default=8192)
+    return ap.parse_args()
+
+
+def cpu_baseline(seq_len: int, d: int, bk: int, topk: int, hkv: int):
+    """The CPU oracle (a PyTorch-eager port of the reference's math) timed on the host cores:
+    forward + backward of the same operator on a bounded sample of the workload."""
+    import torch
+    from fsa_hip.synth import make_qkv, make_topk_idx
+    from oracle import selattn as orc
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    cu = [0, seq_len]
+    q, k, v, do = make_qkv(seq_len, hkv, hkv, d, torch.float32, seed=0)
+    idx = make_topk_idx(cu, hkv, bk, topk, seed=1)
+    _, p_key = orc.count_pairs(idx, bk, cu)
+    flops = 14.0 * d * p_key  # summed over heads already (g = 1)
+    times = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        orc.selected_attention_grads_ref(q, k, v, idx, bk, cu, do)
+        times.append(time.perf_counter() - t0)
+    best = min(times)
+    return {
+        "value": flops / best / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle fwd+bwd (fp32 eager PyTorch), 1 sequence S={seq_len}, Hkv=Hq={hkv}, D={d}, "
+                  f"B_K={bk}, T={topk}; best of 2 runs, {best * 1e3:.0f} ms",
+        "ms": best * 1e3,
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (every box has one GPU); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from fsa.ops.FSA_topk_sparse_attention import (_topk_sparse_attention_bwd_opt,
+                                                   _topk_sparse_attention_fwd_opt)
+    from fsa_hip import _lib, ops
+    from fsa_hip.synth import make_qkv, make_topk_idx
+
+    assert torch.cuda.is_available(), "bench.py needs a ROCm device"
+    dev = torch.device("cuda:0")
+    n, hkv, d, bk, topk = args.seq_len, 4, 128, 64, 16
+    groups = [int(x) for x in args.groups.split(",")]
+    dtype = torch.bfloat16
+    scale = 1.0 / d ** 0.5
+    cu = [0, n]
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    idx_cpu = make_topk_idx(cu, hkv, bk, topk, seed=1)
+    idx = idx_cpu.to(dev)
+    # exact work: valid (query, block) pairs and unmasked (query, key) pairs, summed over kv heads
+    own = torch.arange(n) // bk
+    lo = idx_cpu.long() * bk
+    ok = idx_cpu >= 0
+    nkeys = (torch.minimum(torch.arange(n)[None, :, None], lo + bk - 1) - lo + 1).clamp(min=0)
+    pairs = int(ok.sum())
+    p_key = int(torch.where(ok, nkeys, torch.zeros_like(nkeys)).sum())
+    nblk = (n + bk - 1) // bk
+    del own, lo, ok, nkeys
+
+    data = {}
+    for g in groups:
+        data[g] = tuple(x.to(dev) for x in make_qkv(n, hkv * g, hkv, d, dtype, seed=100 + g))
+
+    def run_g(g):
+        q, k, v, do = data[g]
+        o, lse, perm = _topk_sparse_attention_fwd_opt(q, k, v, idx, bk, cu_t, cu_t, n, n, scale)
+        return _topk_sparse_attention_bwd_opt(o, do, lse, q, k, v, idx, bk, cu_t, cu_t, n, n, scale, perm)
+
+    def step():
+        for g in groups:
+            run_g(g)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    flops_g = {g: 14.0 * d * p_key * g for g in groups}
+    total_tflop = sum(flops_g.values()) / 1e12
+    value = total_tflop / (ms_per_step * 1e-3)
+
+    # per-kernel durations from HIP events recorded on the launch stream inside the library
+    _lib.profile_enable(True)
+    reps = max(3, min(10, args.steps))
+    for _ in range(reps):
+        for g in groups:
+            run_g(g)
+    torch.cuda.synchronize()
+    recs = _lib.profile_records()
+    _lib.profile_enable(False)
+    per_call = len(recs) // (reps * len(groups))
+    kern = {}
+    for i, (name, ms) in enumerate(recs):
+        g = groups[(i // per_call) % len(groups)]
+        kern.setdefault((name, g), []).append(ms)
+    kern = {k_: sum(v_) / len(v_) for k_, v_ in kern.items()}
+
+    e = 2  # bytes per element
+    def algo(name, g):
+        hq = hkv * g
+        fl = {"selattn_fwd_main": 4.0, "selattn_bwd_dq": 6.0, "selattn_bwd_dkdv": 4.0}
+        if name in fl:
+            return "mfma", fl[name] * d * p_key * g
+        if name == "selattn_fwd_reduce":
+            return "hbm", pairs * g * (d * e + 4) + n * hq * (d * e + 4)
+        if name == "selattn_bwd_dq_reduce":
+            return "hbm", pairs * g * d * e + n * hq * d * e
+        if name == "selattn_bwd_delta":
+            return "hbm", 2 * n * hq * d * e + n * hq * 4
+        if name == "index_build":
+            return "hbm", 4 * hkv * n * topk * 2 + 4 * (pairs + 2 * nblk * hkv)
+        if name == "selattn_bwd_dkdv_reduce":
+            return "hbm", 2 * n * hkv * d * e
+        return "hbm", 0.0
+
+    kernels = []
+    for (name, g), ms in sorted(kern.items(), key=lambda kv: -kv[1]):
+        bound, work = algo(name, g)
+        if bound == "mfma":
+            ach, peak, unit = work / (ms * 1e-3) / 1e12, MFMA_PEAK_TFLOPS, "TFLOP/s"
+        else:
+            ach, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
+        kernels.append({"kernel": name, "gqa": g, "ms": round(ms, 4), "bound": bound,
+                        "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)})
+    dom = kernels[0]
+    roofline = {"kernel": f"{dom['kernel']} (GQA {dom['gqa']})", "bound": dom["bound"],
+                "achieved": dom["achieved"], "peak": dom["peak"], "unit": dom["unit"], "frac": dom["frac"],
+                "traffic": None}
+
+    per_gqa = []
+    for g in groups:
+        parts = {nm: ms for (nm, gg), ms in kern.items() if gg == g}
+        fwd = parts.get("selattn_fwd_main", 0) + parts.get("selattn_fwd_reduce", 0)
+        bwd = sum(ms for nm, ms in parts.items() if nm.startswith("selattn_bwd"))
+        tot = fwd + bwd + parts.get("index_build", 0)
+        per_gqa.append({"gqa": g, "hq": hkv * g, "index_ms": round(parts.get("index_build", 0), 4),
+                        "fwd_ms": round(fwd, 4), "bwd_ms": round(bwd, 4),
+                        "tflops": round(flops_g[g] / 1e12 / (tot * 1e-3), 2),
+                        "mfma_frac": round(flops_g[g] / 1e12 / (tot * 1e-3) / MFMA_PEAK_TFLOPS, 4)})
+
+    out = {
+        "metric": METRIC,
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"selected attention index+fwd+bwd, 1 varlen sequence S={n}, Hkv={hkv}, "
+                               f"GQA {'/'.join(map(str, groups))} swept in one step, D={d}, B_K={bk}, T={topk}",
+                   "pairs_per_kv_head": pairs // hkv, "unmasked_qk_pairs_per_q_head": p_key // hkv,
+                   "tflop_per_step": round(total_tflop, 4), "seed": 1},
+        "mfma_frac_whole_step": round(value / MFMA_PEAK_TFLOPS, 4),
+        "roofline": roofline,
+        "per_gqa": per_gqa,
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args.cpu_seq_len, d, bk, topk, hkv)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

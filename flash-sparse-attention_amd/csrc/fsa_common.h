@@ -121,6 +121,15 @@ void set_error(const char* fmt, ...);
     }                                                                        \
   } while (0)
 
+// Optional per-kernel timing: while fsa_profile_enable(1) is in effect every
+// launch wrapped in a ProfScope is bracketed by HIP events on its stream.
+struct ProfScope {
+  ProfScope(const char* name, hipStream_t stream);
+  ~ProfScope();
+  int idx_;
+  hipStream_t stream_;
+};
+
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 }  // namespace fsa

@@ -297,6 +297,7 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
   const int ntiles = (int)((n_items + RS_TILE - 1) / RS_TILE);
   const uint32_t sentinel = (uint32_t)max_blocks;
 
+  ProfScope ps_("index_build", stream);  // the whole pipeline of small kernels as one record
   cu_blocks_kernel<<<1, 64, 0, stream>>>(cu_seqlens, batch, block_size, cu_blocks);
   dim3 g_items((unsigned)((n_items + 255) / 256), num_kv_heads);
   make_keys_kernel<<<g_items, 256, 0, stream>>>(topk_idx, topk_stride_h, topk_stride_n, cu_seqlens,

@@ -529,9 +529,18 @@ static int launch_bwd(const SelBwdParams& pdq, const SelBwdParams& pkv, int hkv,
   if (rc) return rc;
   rc = set_lds(selattn_bwd_dkdv_kernel<T, D, BK>, KvCfg<D, BK>::BYTES);
   if (rc) return rc;
-  selattn_bwd_dq_kernel<T, D, BK><<<dim3((unsigned)tiles_dq, hkv), DQ_THREADS, DqLds<D, BK>::BYTES, stream>>>(pdq);
-  selattn_bwd_dkdv_kernel<T, D, BK><<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES, stream>>>(pkv);
-  selattn_bwd_dkdv_reduce_kernel<T, D, BK><<<dim3((unsigned)pkv.max_blocks, hkv), 256, 0, stream>>>(pkv);
+  {
+    ProfScope ps_("selattn_bwd_dq", stream);
+    selattn_bwd_dq_kernel<T, D, BK><<<dim3((unsigned)tiles_dq, hkv), DQ_THREADS, DqLds<D, BK>::BYTES, stream>>>(pdq);
+  }
+  {
+    ProfScope ps_("selattn_bwd_dkdv", stream);
+    selattn_bwd_dkdv_kernel<T, D, BK><<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES, stream>>>(pkv);
+  }
+  {
+    ProfScope ps_("selattn_bwd_dkdv_reduce", stream);
+    selattn_bwd_dkdv_reduce_kernel<T, D, BK><<<dim3((unsigned)pkv.max_blocks, hkv), 256, 0, stream>>>(pkv);
+  }
   return 0;
 }
 
@@ -565,6 +574,7 @@ static int launch_rowwise(int d, const void* o, int64_t o_sn, int64_t o_sh, cons
   if (d == DD) {                                                                                   \
     constexpr int RPB = 256 / (DD / 8);                                                            \
     const unsigned grid = (unsigned)((rows + RPB - 1) / RPB);                                      \
+    ProfScope ps_(second ? "selattn_bwd_dq_reduce" : "selattn_bwd_delta", stream);                 \
     if (!second)                                                                                   \
       selattn_bwd_delta_kernel<T, DD><<<grid, 256, 0, stream>>>((const T*)o, o_sn, o_sh,           \
                                                                 (const T*)d_o, do_sn, do_sh, n, hq, \

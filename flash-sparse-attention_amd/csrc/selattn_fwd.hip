@@ -310,6 +310,7 @@ static int launch_main(const SelFwdParams& p, int hkv, int64_t max_tiles, hipStr
     attr_done = true;
   }
   dim3 grid((unsigned)max_tiles, hkv);
+  ProfScope ps_("selattn_fwd_main", stream);
   selattn_fwd_main_kernel<T, D, BK><<<grid, SEL_THREADS, lds, stream>>>(p);
   return 0;
 }
@@ -342,6 +343,7 @@ static int launch_reduce(int d, const void* o_part, const float* lse_part, const
 #define FSA_CASE(DD)                                                                          \
   if (d == DD) {                                                                              \
     constexpr int RPB = 256 / (DD / 8);                                                       \
+    ProfScope ps_("selattn_fwd_reduce", stream);                                              \
     selattn_fwd_reduce_kernel<T, DD><<<(unsigned)((rows + RPB - 1) / RPB), 256, 0, stream>>>( \
         (const T*)o_part, lse_part, slot_of, cap, n, hq, g, topk, (T*)o, o_sn, o_sh, lse);    \
     return 0;                                                                                 \

@@ -19,6 +19,9 @@ i32, i64, f32, vp, sz = C.c_int32, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
 SIGNATURES = {
     "fsa_version": (C.c_int, []),
     "fsa_last_error": (C.c_char_p, []),
+    "fsa_profile_enable": (C.c_int, [C.c_int]),
+    "fsa_profile_count": (C.c_int, []),
+    "fsa_profile_get": (C.c_int, [C.c_int, C.c_char_p, C.c_int, C.POINTER(C.c_float)]),
     "fsa_index_workspace_bytes": (sz, [i64, i32, i32, i64]),
     "fsa_build_index": (C.c_int, [vp, i64, i64, vp, i32, i64, i32, i32, i32, i64,
                                   vp, vp, vp, vp, vp, vp, sz, vp]),
@@ -71,3 +74,19 @@ def check(rc: int, what: str):
     if rc < 0:
         raise ValueError(f"{what}: {msg} (code {rc})")
     raise RuntimeError(f"{what}: HIP error {rc}: {msg}")
+
+
+def profile_enable(on: bool):
+    load().fsa_profile_enable(1 if on else 0)
+
+
+def profile_records():
+    """[(label, milliseconds)] of the launches recorded since profile_enable(True)."""
+    lib = load()
+    out = []
+    buf = C.create_string_buffer(128)
+    ms = C.c_float()
+    for i in range(lib.fsa_profile_count()):
+        check(lib.fsa_profile_get(i, buf, 128, C.byref(ms)), "fsa_profile_get")
+        out.append((buf.value.decode(), ms.value))
+    return out

@@ -39,6 +39,15 @@ int fsa_version(void);
 /* Human-readable description of the last error on the calling thread. */
 const char* fsa_last_error(void);
 
+/* Per-kernel timing for benchmarks (replaces the CUDA-event timer of
+ * utils.py:6-27).  While enabled, every kernel launch of the library is
+ * bracketed by HIP events on its stream; fsa_profile_get waits for record i and
+ * returns its label and duration in milliseconds.  fsa_profile_enable(0 or 1)
+ * also discards the records collected so far. */
+int fsa_profile_enable(int on);
+int fsa_profile_count(void);
+int fsa_profile_get(int i, char* name, int name_cap, float* ms);
+
 /* ------------------------------------------------------------------------
  * Inverted block->query index.
  * Replaces: torch.bincount + build_block_to_token_triton + boolean compaction

@@ -10,8 +10,9 @@ Pinning status (tests/test_oracle_selattn.py):
   selected_attention_ref : pinned - dense-mask fp64 softmax, SDPA with an
       explicit bool mask, closed forms (token 0, all-blocks == causal,
       own-block only == block-diagonal causal), slot-permutation invariance.
-  selected_attention_grads_ref : pinned - autograd of the dense fp64
-      formulation and central finite differences on tiny inputs.
+  selected_attention_grads_ref : pinned - explicit backward formulas checked
+      against autograd of the dense fp64 formulation, autograd of
+      selected_attention_ref and central finite differences on tiny inputs.
   build_index_ref : pinned - brute-force Python loops, torch.bincount,
       exclusive cumsum identity.
 """
@@ -64,51 +65,108 @@ def selected_attention_ref(
     o_chunks = []
     lse_chunks = []
     ar = torch.arange(block_size)
+    B = block_size
     for (s0, s1) in _seq_bounds(cu_seqlens):
         L = s1 - s0
-        ks, vs = kf[s0:s1], vf[s0:s1]
+        nblk = (L + B - 1) // B
+        pad = nblk * B - L
+        # [Hkv, nblk, B*D] block views of this sequence's keys / values (zero padded tail)
+        kb = torch.nn.functional.pad(kf[s0:s1], (0, 0, 0, 0, 0, pad)).reshape(nblk, B, Hkv, D).permute(2, 0, 1, 3).reshape(Hkv, nblk, B * D)
+        vb = torch.nn.functional.pad(vf[s0:s1], (0, 0, 0, 0, 0, pad)).reshape(nblk, B, Hkv, D).permute(2, 0, 1, 3).reshape(Hkv, nblk, B * D)
         for i0 in range(0, L, q_chunk):
             i1 = min(L, i0 + q_chunk)
             C = i1 - i0
             idx = topk_idx[:, s0 + i0 : s0 + i1, :].long()  # [Hkv, C, T]
-            kpos = idx[..., None] * block_size + ar  # [Hkv, C, T, B]
+            kpos = idx[..., None] * B + ar  # [Hkv, C, T, B]
             qpos = torch.arange(i0, i1)[None, :, None, None]
-            valid = (idx[..., None] >= 0) & (kpos <= qpos) & (kpos < L)
-            kpos = kpos.clamp(0, L - 1).reshape(Hkv, C, T * block_size)
-            valid = valid.reshape(Hkv, C, T * block_size)
-            hsel = torch.arange(Hkv)[:, None, None]
-            kg = ks[kpos, hsel]  # [Hkv, C, TB, D]
-            vg = vs[kpos, hsel]
-            qc = qf[s0 + i0 : s0 + i1].reshape(C, Hkv, g, D).permute(1, 0, 2, 3)  # [Hkv, C, g, D]
-            s = torch.einsum("hcgd,hckd->hcgk", qc, kg) * c
-            s = s.masked_fill(~valid[:, :, None, :], float("-inf"))
-            m = s.max(dim=-1, keepdim=True).values
-            m = torch.where(torch.isinf(m), torch.zeros_like(m), m)
-            p = torch.exp2(s - m)
-            l = p.sum(-1, keepdim=True)
-            lse = (m + torch.log2(l)).squeeze(-1)  # [Hkv, C, g]
-            o = torch.einsum("hcgk,hckd->hcgd", p / l, vg)
-            o_chunks.append(o.permute(1, 0, 2, 3).reshape(C, Hq, D))
-            lse_chunks.append(lse.permute(0, 2, 1).reshape(Hq, C))
+            valid = ((idx[..., None] >= 0) & (idx[..., None] < nblk) & (kpos <= qpos) & (kpos < L))
+            valid = valid.reshape(Hkv, C, T * B)
+            bsel = idx.clamp(0, nblk - 1).reshape(Hkv, C * T)
+            qc = qf[s0 + i0 : s0 + i1].reshape(C, Hkv, g, D)
+            o_h, lse_h = [], []
+            for kh in range(Hkv):
+                kg = kb[kh].index_select(0, bsel[kh]).reshape(C, T * B, D)
+                vg = vb[kh].index_select(0, bsel[kh]).reshape(C, T * B, D)
+                s = torch.bmm(qc[:, kh], kg.transpose(1, 2)) * c  # [C, g, TB]
+                s = s.masked_fill(~valid[kh][:, None, :], float("-inf"))
+                m = s.max(dim=-1, keepdim=True).values
+                m = torch.where(torch.isinf(m), torch.zeros_like(m), m)
+                p = torch.exp2(s - m)
+                l = p.sum(-1, keepdim=True)
+                lse_h.append((m + torch.log2(l)).squeeze(-1))  # [C, g]
+                o_h.append(torch.bmm(p / l, vg))  # [C, g, D]
+            o_chunks.append(torch.stack(o_h, 1).reshape(C, Hq, D))
+            lse_chunks.append(torch.stack(lse_h, 1).reshape(C, Hq).t())
     return torch.cat(o_chunks, 0), torch.cat(lse_chunks, 1)
 
 
 def selected_attention_grads_ref(q, k, v, topk_idx, block_size, cu_seqlens, do, softmax_scale=None,
                                  dtype=torch.float32, q_chunk: int = 128):
-    """(O, LSE2, dQ, dK, dV) through autograd of `selected_attention_ref`.
+    """(O, LSE2, dQ, dK, dV) by the explicit backward formulas, chunk by chunk.
 
-    Mathematically the formulas of FSA_topk_sparse_attention.py:1229-1237 and
-    :1697-1709: dS = scale * P * (dP - delta), dQ = dS K, dK = sum over the
-    group's heads of dS^T Q, dV = sum over heads of P^T dO
-    (dK/dV head sum: FSA_topk_sparse_attention.py:1854-1855).
+    FSA_topk_sparse_attention.py:1229-1237 and :1697-1709 with P = 2^(s - LSE2):
+    delta = sum_d O dO, dP = dO V^T, dS = scale * P * (dP - delta), dQ = dS K,
+    dK = sum over the group's heads of dS^T Q, dV = sum over heads of P^T dO
+    (dK/dV head sum: :1854-1855).  No autograd, so memory stays bounded; the
+    formulas themselves are checked against autograd of the dense formulation
+    and finite differences in the tests.
     """
-    q_ = q.detach().to(dtype).requires_grad_(True)
-    k_ = k.detach().to(dtype).requires_grad_(True)
-    v_ = v.detach().to(dtype).requires_grad_(True)
-    o, lse = selected_attention_ref(q_, k_, v_, topk_idx, block_size, cu_seqlens, softmax_scale,
-                                    q_chunk=q_chunk, dtype=dtype)
-    (o * do.to(dtype)).sum().backward()
-    return o.detach(), lse.detach(), q_.grad, k_.grad, v_.grad
+    N, Hq, D = q.shape
+    Hkv = k.shape[1]
+    g = Hq // Hkv
+    T = topk_idx.shape[-1]
+    B = block_size
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    c = softmax_scale * LOG2E
+    qf, kf, vf, dof = (x.detach().to(dtype) for x in (q, k, v, do))
+    o_out = torch.empty_like(qf)
+    lse_out = torch.empty(Hq, N, dtype=dtype)
+    dq = torch.empty_like(qf)
+    dk = torch.zeros_like(kf)
+    dv = torch.zeros_like(vf)
+    ar = torch.arange(B)
+    for (s0, s1) in _seq_bounds(cu_seqlens):
+        L = s1 - s0
+        if L == 0:
+            continue
+        nblk = (L + B - 1) // B
+        pad = nblk * B - L
+        kb = torch.nn.functional.pad(kf[s0:s1], (0, 0, 0, 0, 0, pad)).reshape(nblk, B, Hkv, D).permute(2, 0, 1, 3).reshape(Hkv, nblk, B * D)
+        vb = torch.nn.functional.pad(vf[s0:s1], (0, 0, 0, 0, 0, pad)).reshape(nblk, B, Hkv, D).permute(2, 0, 1, 3).reshape(Hkv, nblk, B * D)
+        dkb = torch.zeros_like(kb)
+        dvb = torch.zeros_like(vb)
+        for i0 in range(0, L, q_chunk):
+            i1 = min(L, i0 + q_chunk)
+            C = i1 - i0
+            idx = topk_idx[:, s0 + i0 : s0 + i1, :].long()
+            kpos = idx[..., None] * B + ar
+            qpos = torch.arange(i0, i1)[None, :, None, None]
+            valid = ((idx[..., None] >= 0) & (idx[..., None] < nblk) & (kpos <= qpos) & (kpos < L))
+            valid = valid.reshape(Hkv, C, T * B)
+            bsel = idx.clamp(0, nblk - 1).reshape(Hkv, C * T)
+            qc = qf[s0 + i0 : s0 + i1].reshape(C, Hkv, g, D)
+            doc = dof[s0 + i0 : s0 + i1].reshape(C, Hkv, g, D)
+            for kh in range(Hkv):
+                kg = kb[kh].index_select(0, bsel[kh]).reshape(C, T * B, D)
+                vg = vb[kh].index_select(0, bsel[kh]).reshape(C, T * B, D)
+                s = torch.bmm(qc[:, kh], kg.transpose(1, 2)) * c
+                s = s.masked_fill(~valid[kh][:, None, :], float("-inf"))
+                lse = torch.logsumexp(s * (1.0 / LOG2E), dim=-1, keepdim=True) * LOG2E  # base 2
+                p = torch.exp2(s - lse)
+                o = torch.bmm(p, vg)
+                dp = torch.bmm(doc[:, kh], vg.transpose(1, 2))
+                delta = (o * doc[:, kh]).sum(-1, keepdim=True)
+                ds = softmax_scale * p * (dp - delta)
+                hs = slice(kh * g, (kh + 1) * g)
+                o_out[s0 + i0 : s0 + i1, hs] = o
+                lse_out[hs, s0 + i0 : s0 + i1] = lse.squeeze(-1).t()
+                dq[s0 + i0 : s0 + i1, hs] = torch.bmm(ds, kg)
+                dkb[kh].index_add_(0, bsel[kh], torch.bmm(ds.transpose(1, 2), qc[:, kh]).reshape(C * T, B * D))
+                dvb[kh].index_add_(0, bsel[kh], torch.bmm(p.transpose(1, 2), doc[:, kh]).reshape(C * T, B * D))
+        dk[s0:s1] = dkb.reshape(Hkv, nblk * B, D)[:, :L].permute(1, 0, 2)
+        dv[s0:s1] = dvb.reshape(Hkv, nblk * B, D)[:, :L].permute(1, 0, 2)
+    return o_out, lse_out, dq, dk, dv
 
 
 def dense_mask(topk_idx: torch.Tensor, block_size: int, cu_seqlens) -> torch.Tensor:

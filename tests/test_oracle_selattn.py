@@ -96,6 +96,13 @@ def test_grads_match_dense_autograd_and_finite_differences():
     assert torch.allclose(dq, qd.grad, atol=1e-11)
     assert torch.allclose(dk, kd.grad, atol=1e-11)
     assert torch.allclose(dv, vd.grad, atol=1e-11)
+    assert torch.allclose(o, od, atol=1e-12)
+    # and against autograd through the gather formulation
+    qg, kg, vg = (x.clone().requires_grad_(True) for x in (q, k, v))
+    og, lseg = orc.selected_attention_ref(qg, kg, vg, topk, 8, cu, dtype=torch.float64)
+    (og * do).sum().backward()
+    assert torch.allclose(dq, qg.grad, atol=1e-11) and torch.allclose(dk, kg.grad, atol=1e-11)
+    assert torch.allclose(dv, vg.grad, atol=1e-11) and torch.allclose(lse, lseg, atol=1e-11)
 
     def loss(q_, k_, v_):
         return float((orc.selected_attention_ref(q_, k_, v_, topk, 8, cu, dtype=torch.float64)[0] * do).sum())
