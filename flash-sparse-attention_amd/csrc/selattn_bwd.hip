@@ -259,11 +259,12 @@ template <int D, int BK> struct KvCfg {
   static constexpr int CPT = KV_R * CPR / NT;  // chunks per thread and tensor
   static constexpr int ROW_STEP = NT / CPR;
   static constexpr int BYTES = 2 * KV_R * QS * 2 + KV_R * 12;
+  static constexpr int MIN_WAVES = (D <= 128 && NT <= 256) ? 2 : 1;  // work-groups per CU the registers allow
   static_assert(KV_R * CPR % NT == 0, "tile must divide evenly over the threads");
 };
 
 template <typename T, int D, int BK>
-__global__ void __launch_bounds__((KvCfg<D, BK>::NT))
+__global__ void __launch_bounds__((KvCfg<D, BK>::NT), (KvCfg<D, BK>::MIN_WAVES))
 selattn_bwd_dkdv_kernel(SelBwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
@@ -321,7 +322,16 @@ selattn_bwd_dkdv_kernel(SelBwdParams p) {
   vec8 qst[C::CPT], dost[C::CPT];
   float lse_st = 0.f, del_st = 0.f;
   int lim_st = 0;
-  // global -> registers for the pass starting at row `base`
+  int tok_pf[C::CPT], tok_stat = 0;  // token ids of the pass after the one being fetched
+  auto fetch_tokens = [&](int base) {
+#pragma unroll
+    for (int j = 0; j < C::CPT; ++j) {
+      const int r = base + ld_row + C::ROW_STEP * j;
+      tok_pf[j] = r < row_hi ? toks[r / p.g] : 0;
+    }
+    if (tid < KV_R) tok_stat = base + tid < row_hi ? toks[(base + tid) / p.g] : 0;
+  };
+  // global -> registers for the pass starting at row `base` (its token ids are in tok_pf)
   auto fetch = [&](int base) {
 #pragma unroll
     for (int j = 0; j < C::CPT; ++j) {
@@ -330,7 +340,7 @@ selattn_bwd_dkdv_kernel(SelBwdParams p) {
       dost[j] = zero8<T>();
       if (r < row_hi) {
         const int trank = r / p.g, head = r - trank * p.g;
-        const int token = toks[trank];
+        const int token = tok_pf[j];
         qst[j] = load16<vec8>(qbase + (int64_t)token * p.q_sn + (int64_t)head * p.q_sh + ld_col * 8);
         dost[j] = load16<vec8>(dobase + (int64_t)token * p.do_sn + (int64_t)head * p.do_sh + ld_col * 8);
       }
@@ -342,7 +352,7 @@ selattn_bwd_dkdv_kernel(SelBwdParams p) {
       lim_st = -1;
       if (r < row_hi) {
         const int trank = r / p.g, head = r - trank * p.g;
-        const int token = toks[trank];
+        const int token = tok_stat;
         const int64_t stat = (int64_t)(h * p.g + head) * p.n_tokens + token;
         lse_st = p.lse[stat];
         del_st = p.delta[stat];
@@ -377,12 +387,17 @@ selattn_bwd_dkdv_kernel(SelBwdParams p) {
   const int a_off = l16 * QS + 8 * kg;                            // + rt*16*QS + 32*s
   const int tr_off = (4 * kg + (l16 >> 2)) * QS + 4 * (l16 & 3);  // + 32*u*QS + 16*dtile
 
+  fetch_tokens(row_lo);
   fetch(row_lo);
+  fetch_tokens(row_lo + KV_R);
   stash();
   __syncthreads();
   for (int base = row_lo; base < row_hi; base += KV_R) {
     const bool more = base + KV_R < row_hi;
-    if (more) fetch(base + KV_R);
+    if (more) {
+      fetch(base + KV_R);
+      fetch_tokens(base + 2 * KV_R);
+    }
 
     vec4 pk[NRT], dsk[NRT];
 #pragma unroll
