@@ -1,0 +1,341 @@
+// dK/dV kernel shared by selected attention (gathered query rows of a kv block)
+// and compressed attention (the dense range of queries that can see a tile of
+// compressed keys).  Block-major, contraction over the rows: each wave owns 16
+// keys and keeps their K / V fragments in registers; Q / dO tiles of 64 rows go
+// through LDS once and feed S = Q K^T, dP = dO V^T (16x16x32 MFMA) and, through
+// transposing LDS reads, dV^T += dO^T P and dK^T += Q^T dS.  The g heads of a
+// group are rows of the same tile, so the results are already summed over the
+// group, in fp32.  A block whose rows span several work-groups writes fp32
+// partials that the reduce kernel adds in a fixed order.
+#pragma once
+#include "fsa_common.h"
+
+namespace fsa {
+
+struct SelBwdParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* d_o;
+  const float* lse;    // [Hq, N]
+  const float* delta;  // [Hq, N]
+  int64_t q_sn, q_sh, k_sn, k_sh, v_sn, v_sh, do_sn, do_sh;
+  const int32_t* cu_seqlens;
+  const int32_t* cu_blocks;
+  const int32_t* counts;
+  const int32_t* starts;
+  const int32_t* sel_tokens;
+  const int32_t* tile_prefix;
+  int batch;
+  int64_t max_blocks;
+  int64_t cap;
+  int64_t n_tokens;
+  int g;
+  float scale;
+  float scale_log2;
+  void* dq_part;     // [Hkv, cap, g, D] lane-native order
+  float* dkdv_part;  // [Hkv, max_tiles, 2, BK, D]
+  int64_t max_tiles;
+  void* dk;          // rows of k's shape, strides dk_sn / dk_sh
+  void* dv;
+  int64_t dk_sn, dk_sh;
+  // compressed-attention mode only
+  const int32_t* cu_seqlens_k;
+  int kernel_size, kernel_stride;
+};
+
+
+constexpr int KV_MODE_SELECTED = 0;
+constexpr int KV_MODE_COMPRESSED = 1;
+
+// What a "block" of the work list is in each mode.
+template <int MODE, int BK> struct KvBlock {
+  int seq_start, q_first, key_row0, n_keys_valid, key_base;
+  __device__ __forceinline__ void init(const SelBwdParams& p, int gb) {
+    const int s = upper_seg(p.cu_blocks, p.batch, gb);
+    const int b_local = gb - p.cu_blocks[s];
+    seq_start = p.cu_seqlens[s];
+    if (MODE == KV_MODE_SELECTED) {
+      key_row0 = seq_start + b_local * BK;                 // K/V rows are tokens
+      n_keys_valid = p.cu_seqlens[s + 1] - key_row0;       // may exceed BK
+      q_first = 0;
+      key_base = b_local * BK;                             // position of key 0 of the block
+    } else {
+      const int k0 = p.cu_seqlens_k[s];
+      key_row0 = k0 + b_local * BK;                        // K/V rows are compressed tokens
+      n_keys_valid = p.cu_seqlens_k[s + 1] - key_row0;
+      q_first = b_local * BK * p.kernel_stride + p.kernel_size - 1;  // first query that sees key 0
+      key_base = b_local * BK;
+    }
+  }
+  // number of keys of the block visible to the query at sequence-local position qpos, minus one
+  __device__ __forceinline__ int limit(const SelBwdParams& p, int qpos) const {
+    if (MODE == KV_MODE_SELECTED) return qpos - key_base;
+    return (qpos - p.kernel_size + 1) / p.kernel_stride - key_base;  // qpos >= q_first >= ks-1
+  }
+};
+
+// ----------------------------------------------------------------- dkdv ----
+constexpr int KV_R = 64;             // gathered rows per pass
+constexpr int KV_TILE_ROWS = 4096;   // rows per work-group
+
+template <int D, int BK> struct KvCfg {
+  static constexpr int NW = BK / 16;        // one wave per 16 keys
+  static constexpr int NT = NW * 64;
+  static constexpr int QS = D + 8;          // LDS row stride of the Q / dO tiles
+  static constexpr int CPR = D / 8;         // 16-byte chunks per row
+  static constexpr int CPT = KV_R * CPR / NT;  // chunks per thread and tensor
+  static constexpr int ROW_STEP = NT / CPR;
+  static constexpr int BYTES = 2 * KV_R * QS * 2 + KV_R * 12;
+  static constexpr int MIN_WAVES = (D <= 128 && NT <= 256) ? 2 : 1;  // work-groups per CU the registers allow
+  static_assert(KV_R * CPR % NT == 0, "tile must divide evenly over the threads");
+};
+
+template <typename T, int D, int BK, int MODE>
+__global__ void __launch_bounds__((KvCfg<D, BK>::NT), (KvCfg<D, BK>::MIN_WAVES))
+attn_bwd_dkdv_kernel(SelBwdParams p) {
+  typedef typename Elem<T>::vec8 vec8;
+  typedef typename Elem<T>::vec4 vec4;
+  typedef KvCfg<D, BK> C;
+  constexpr int QS = C::QS, NS = D / 32, NDT = D / 16, NRT = KV_R / 16, NU = KV_R / 32;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T* Qs = reinterpret_cast<T*>(smem);
+  T* Os = Qs + KV_R * QS;
+  float* lse_s = reinterpret_cast<float*>(Os + KV_R * QS);
+  float* del_s = lse_s + KV_R;
+  int* lim_s = reinterpret_cast<int*>(del_s + KV_R);
+
+  const int h = blockIdx.y;
+  const int64_t nbp1 = p.max_blocks + 1;
+  const int32_t* tp = p.tile_prefix + h * nbp1;
+  const int w = blockIdx.x;
+  if (w >= tp[p.max_blocks]) return;
+  const int gb = upper_seg(tp, (int)p.max_blocks, w);
+  KvBlock<MODE, BK> blk;
+  blk.init(p, gb);
+  const int rows = p.counts[h * p.max_blocks + gb] * p.g;
+  const int start = MODE == KV_MODE_SELECTED ? p.starts[h * nbp1 + gb] : 0;
+  const int ntile_b = tp[gb + 1] - tp[gb];
+  const int row_lo = (w - tp[gb]) * KV_TILE_ROWS;
+  const int row_hi = min(rows, row_lo + KV_TILE_ROWS);
+
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int l16 = lane & 15, kg = lane >> 4;
+  const int key = wv * 16 + l16;       // this lane's key inside the block (B operand column)
+  const int ktok = blk.key_row0 + key;  // row of this lane's key in k / v
+  const bool key_ok = key < blk.n_keys_valid;
+
+  // K / V fragments of this wave's 16 keys stay in registers: B[k = d][n = key]
+  vec8 kf[NS], vf[NS];
+  {
+    const T* krow = reinterpret_cast<const T*>(p.k) + (int64_t)ktok * p.k_sn + (int64_t)h * p.k_sh + 8 * kg;
+    const T* vrow = reinterpret_cast<const T*>(p.v) + (int64_t)ktok * p.v_sn + (int64_t)h * p.v_sh + 8 * kg;
+#pragma unroll
+    for (int s_ = 0; s_ < NS; ++s_) {
+      kf[s_] = zero8<T>();
+      vf[s_] = zero8<T>();
+      if (key_ok) {
+        kf[s_] = load16<vec8>(krow + 32 * s_);
+        vf[s_] = load16<vec8>(vrow + 32 * s_);
+      }
+    }
+  }
+
+  const int32_t* toks = MODE == KV_MODE_SELECTED ? p.sel_tokens + (int64_t)h * p.cap + start : nullptr;
+  // row r of the block -> global query row
+  auto row_token = [&](int r) {
+    if (MODE == KV_MODE_SELECTED) return (int)toks[r / p.g];
+    return blk.seq_start + blk.q_first + r / p.g;
+  };
+  const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)h * p.g * p.q_sh;
+  const T* dobase = reinterpret_cast<const T*>(p.d_o) + (int64_t)h * p.g * p.do_sh;
+  const int ld_row = tid / C::CPR, ld_col = tid % C::CPR;
+
+  vec8 qst[C::CPT], dost[C::CPT];
+  float lse_st = 0.f, del_st = 0.f;
+  int lim_st = 0;
+  int tok_pf[C::CPT], tok_stat = 0;  // token ids of the pass after the one being fetched
+  auto fetch_tokens = [&](int base) {
+#pragma unroll
+    for (int j = 0; j < C::CPT; ++j) {
+      const int r = base + ld_row + C::ROW_STEP * j;
+      tok_pf[j] = r < row_hi ? row_token(r) : 0;
+    }
+    if (tid < KV_R) tok_stat = base + tid < row_hi ? row_token(base + tid) : 0;
+  };
+  // global -> registers for the pass starting at row `base` (its token ids are in tok_pf)
+  auto fetch = [&](int base) {
+#pragma unroll
+    for (int j = 0; j < C::CPT; ++j) {
+      const int r = base + ld_row + C::ROW_STEP * j;
+      qst[j] = zero8<T>();
+      dost[j] = zero8<T>();
+      if (r < row_hi) {
+        const int trank = r / p.g, head = r - trank * p.g;
+        const int token = tok_pf[j];
+        qst[j] = load16<vec8>(qbase + (int64_t)token * p.q_sn + (int64_t)head * p.q_sh + ld_col * 8);
+        dost[j] = load16<vec8>(dobase + (int64_t)token * p.do_sn + (int64_t)head * p.do_sh + ld_col * 8);
+      }
+    }
+    if (tid < KV_R) {
+      const int r = base + tid;
+      lse_st = INFINITY;  // rows past the end: P = exp2(s - inf) = 0
+      del_st = 0.f;
+      lim_st = -1;
+      if (r < row_hi) {
+        const int trank = r / p.g, head = r - trank * p.g;
+        const int token = tok_stat;
+        const int64_t stat = (int64_t)(h * p.g + head) * p.n_tokens + token;
+        lse_st = p.lse[stat];
+        del_st = p.delta[stat];
+        lim_st = blk.limit(p, token - blk.seq_start);
+      }
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int j = 0; j < C::CPT; ++j) {
+      const int row = ld_row + C::ROW_STEP * j;
+      store16(&Qs[row * QS + ld_col * 8], qst[j]);
+      store16(&Os[row * QS + ld_col * 8], dost[j]);
+    }
+    if (tid < KV_R) {
+      lse_s[tid] = lse_st;
+      del_s[tid] = del_st;
+      lim_s[tid] = lim_st;
+    }
+  };
+
+  f32x4 dkacc[NDT], dvacc[NDT];
+#pragma unroll
+  for (int t = 0; t < NDT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dkacc[t][i] = 0.f;
+      dvacc[t][i] = 0.f;
+    }
+
+  // lane addresses: A operand rows (natural) and transposing reads
+  const int a_off = l16 * QS + 8 * kg;                            // + rt*16*QS + 32*s
+  const int tr_off = (4 * kg + (l16 >> 2)) * QS + 4 * (l16 & 3);  // + 32*u*QS + 16*dtile
+
+  fetch_tokens(row_lo);
+  fetch(row_lo);
+  fetch_tokens(row_lo + KV_R);
+  stash();
+  __syncthreads();
+  for (int base = row_lo; base < row_hi; base += KV_R) {
+    const bool more = base + KV_R < row_hi;
+    if (more) {
+      fetch(base + KV_R);
+      fetch_tokens(base + 2 * KV_R);
+    }
+
+    vec4 pk[NRT], dsk[NRT];
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt) {
+      f32x4 sacc = {0.f, 0.f, 0.f, 0.f}, dpacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s_ = 0; s_ < NS; ++s_) {
+        vec8 qa = load16<vec8>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
+        sacc = Elem<T>::mfma16(qa, kf[s_], sacc);
+        vec8 da = load16<vec8>(&Os[rt * 16 * QS + a_off + 32 * s_]);
+        dpacc = Elem<T>::mfma16(da, vf[s_], dpacc);
+      }
+      const float4 lse4 = *reinterpret_cast<const float4*>(&lse_s[rt * 16 + 4 * kg]);
+      const float4 del4 = *reinterpret_cast<const float4*>(&del_s[rt * 16 + 4 * kg]);
+      const int4 lim4 = *reinterpret_cast<const int4*>(&lim_s[rt * 16 + 4 * kg]);
+      const float lse_r[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
+      const float del_r[4] = {del4.x, del4.y, del4.z, del4.w};
+      const int lim_r[4] = {lim4.x, lim4.y, lim4.z, lim4.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = key <= lim_r[i] ? exp2f(sacc[i] * p.scale_log2 - lse_r[i]) : 0.f;
+        const float ds = pv * (dpacc[i] - del_r[i]) * p.scale;
+        pk[rt][i] = (T)pv;
+        dsk[rt][i] = (T)ds;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      vec8 pb = __builtin_shufflevector(pk[2 * u], pk[2 * u + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+      vec8 dsb = __builtin_shufflevector(dsk[2 * u], dsk[2 * u + 1], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+      for (int t = 0; t < NDT; ++t) {
+        vec8 doa = lds_read_tr8<T>(&Os[32 * u * QS + tr_off + 16 * t], 16 * QS);
+        dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
+        vec8 qa = lds_read_tr8<T>(&Qs[32 * u * QS + tr_off + 16 * t], 16 * QS);
+        dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
+      }
+    }
+    __syncthreads();
+    if (more) {
+      stash();
+      __syncthreads();
+    }
+  }
+
+  // accumulators: dV^T[d = 16*t + 4*kg + i][key]
+  if (ntile_b == 1) {
+    if (key_ok) {
+      T* dkrow = reinterpret_cast<T*>(p.dk) + (int64_t)ktok * p.dk_sn + (int64_t)h * p.dk_sh + 4 * kg;
+      T* dvrow = reinterpret_cast<T*>(p.dv) + (int64_t)ktok * p.dk_sn + (int64_t)h * p.dk_sh + 4 * kg;
+#pragma unroll
+      for (int t = 0; t < NDT; ++t) {
+        vec4 a, b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          a[i] = (T)dkacc[t][i];
+          b[i] = (T)dvacc[t][i];
+        }
+        store8(dkrow + 16 * t, a);
+        store8(dvrow + 16 * t, b);
+      }
+    }
+  } else {
+    float* part = p.dkdv_part + ((int64_t)h * p.max_tiles + w) * (2 * BK * D) + key * D + 4 * kg;
+#pragma unroll
+    for (int t = 0; t < NDT; ++t) {
+      *reinterpret_cast<f32x4*>(part + 16 * t) = dkacc[t];
+      *reinterpret_cast<f32x4*>(part + BK * D + 16 * t) = dvacc[t];
+    }
+  }
+}
+
+// Blocks with no selecting query get zeros; blocks split over several
+// work-groups get the fixed-order sum of their fp32 partials.
+template <typename T, int D, int BK, int MODE>
+__global__ void __launch_bounds__(256)
+attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
+  typedef typename Elem<T>::vec4 vec4;
+  const int h = blockIdx.y;
+  const int gb = blockIdx.x;
+  if (gb >= p.cu_blocks[p.batch]) return;
+  const int32_t* tp = p.tile_prefix + h * (p.max_blocks + 1);
+  const int t0 = tp[gb], nt = tp[gb + 1] - t0;
+  if (nt == 1) return;
+  KvBlock<MODE, BK> blk;
+  blk.init(p, gb);
+  for (int c = threadIdx.x; c < BK * (D / 4); c += 256) {
+    const int key = c / (D / 4), d4 = (c % (D / 4)) * 4;
+    const int tok = blk.key_row0 + key;
+    if (key >= blk.n_keys_valid) continue;
+    f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = {0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < nt; ++t) {
+      const float* part = p.dkdv_part + ((int64_t)h * p.max_tiles + t0 + t) * (2 * BK * D) + key * D + d4;
+      sk += *reinterpret_cast<const f32x4*>(part);
+      sv += *reinterpret_cast<const f32x4*>(part + BK * D);
+    }
+    vec4 a, b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a[i] = (T)sk[i];
+      b[i] = (T)sv[i];
+    }
+    store8(reinterpret_cast<T*>(p.dk) + (int64_t)tok * p.dk_sn + (int64_t)h * p.dk_sh + d4, a);
+    store8(reinterpret_cast<T*>(p.dv) + (int64_t)tok * p.dk_sn + (int64_t)h * p.dk_sh + d4, b);
+  }
+}
+
+
+}  // namespace fsa

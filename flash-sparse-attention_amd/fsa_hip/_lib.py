@@ -38,6 +38,18 @@ SIGNATURES = {
                                   vp, i32, i64, i32, i32, i32, i32, i32, i64, f32,
                                   vp, vp, vp, vp, vp,
                                   vp, vp, vp, vp, sz, vp]),
+    "fsa_cmpattn_fwd": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64,
+                                  vp, vp, i32, i64, i64, i32, i32, i32, i32, i32, f32,
+                                  vp, i64, i64, vp, vp]),
+    "fsa_cmpattn_bwd_workspace_bytes": (sz, [i64, i64, i64, i32, i32, i32, i32]),
+    "fsa_cmpattn_bwd": (C.c_int, [vp, vp, vp, vp, vp, vp, i32,
+                                  i64, i64, i64, i64, i64, i64, i64, i64, i64, i64,
+                                  vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, i32, f32,
+                                  vp, vp, vp, vp, sz, vp]),
+    "fsa_cmp_topk_workspace_bytes": (sz, [i64, i32, i64]),
+    "fsa_cmp_topk": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, vp, vp, i32,
+                               i64, i64, i64, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, f32,
+                               vp, vp, vp, sz, vp]),
 }
 
 

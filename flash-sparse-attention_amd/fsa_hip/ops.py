@@ -144,3 +144,88 @@ def selattn_bwd(q, k, v, o, do, lse, index: SelIndex, softmax_scale: Optional[fl
         _ptr(dq), _ptr(dk), _ptr(dv), _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_selattn_bwd")
     return dq, dk, dv
+
+
+def _check_cmp(q, ck, cv, cu_q, cu_k):
+    _require_cuda(q, ck, cv, cu_q, cu_k)
+    assert q.dtype in _DTYPE and q.dtype == ck.dtype == cv.dtype
+    assert cu_q.dtype == torch.int32 and cu_k.dtype == torch.int32
+    assert q.stride(2) == 1 and ck.stride(2) == 1 and cv.stride(2) == 1
+    assert ck.shape == cv.shape and q.shape[1] % ck.shape[1] == 0 and q.shape[2] == ck.shape[2]
+
+
+def cmpattn_fwd(q, ck, cv, kernel_size, kernel_stride, cu_q, cu_k, max_seqlen_q, softmax_scale=None):
+    """Compressed attention forward: (o [N,Hq,D], lse [Hq,N] fp32 base 2)."""
+    _check_cmp(q, ck, cv, cu_q, cu_k)
+    lib = _lib.load()
+    n, hq, d = q.shape
+    hkv = ck.shape[1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    o = torch.empty_like(q)
+    lse = torch.empty((hq, n), dtype=torch.float32, device=q.device)
+    if ck.shape[0] == 0:
+        return o.zero_(), lse.fill_(float("-inf"))
+    rc = lib.fsa_cmpattn_fwd(_ptr(q), _ptr(ck), _ptr(cv), _DTYPE[q.dtype], q.stride(0), q.stride(1),
+                             ck.stride(0), ck.stride(1), cv.stride(0), cv.stride(1), _ptr(cu_q), _ptr(cu_k),
+                             cu_q.numel() - 1, n, int(max_seqlen_q), hq, hkv, d, kernel_size, kernel_stride,
+                             float(softmax_scale), _ptr(o), o.stride(0), o.stride(1), _ptr(lse),
+                             _stream(q.device))
+    _lib.check(rc, "fsa_cmpattn_fwd")
+    return o, lse
+
+
+def cmpattn_bwd(q, ck, cv, o, do, lse, kernel_size, kernel_stride, cu_q, cu_k, max_seqlen_q,
+                softmax_scale=None):
+    """Compressed attention backward: (dq, dck, dcv)."""
+    _check_cmp(q, ck, cv, cu_q, cu_k)
+    lib = _lib.load()
+    n, hq, d = q.shape
+    nk, hkv, _ = ck.shape
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if do.stride(2) != 1:
+        do = do.contiguous()
+    dq = torch.empty((n, hq, d), dtype=q.dtype, device=q.device)
+    dck = torch.empty((nk, hkv, d), dtype=q.dtype, device=q.device)
+    dcv = torch.empty((nk, hkv, d), dtype=q.dtype, device=q.device)
+    if nk == 0:
+        return dq.zero_(), dck, dcv
+    batch = cu_q.numel() - 1
+    ws_bytes = lib.fsa_cmpattn_bwd_workspace_bytes(n, nk, int(max_seqlen_q), batch, hq, hkv, d)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    rc = lib.fsa_cmpattn_bwd(_ptr(q), _ptr(ck), _ptr(cv), _ptr(o), _ptr(do), _ptr(lse), _DTYPE[q.dtype],
+                             q.stride(0), q.stride(1), ck.stride(0), ck.stride(1), cv.stride(0), cv.stride(1),
+                             o.stride(0), o.stride(1), do.stride(0), do.stride(1), _ptr(cu_q), _ptr(cu_k),
+                             batch, n, nk, int(max_seqlen_q), hq, hkv, d, kernel_size, kernel_stride,
+                             float(softmax_scale), _ptr(dq), _ptr(dck), _ptr(dcv), _ptr(ws), ws_bytes,
+                             _stream(q.device))
+    _lib.check(rc, "fsa_cmpattn_bwd")
+    return dq, dck, dcv
+
+
+def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_k, max_seqlen_q,
+             max_seqlen_k, init_blocks=1, local_blocks=2, softmax_scale=None, scores_to_bf16=True,
+             return_block_score=False):
+    """Top-k block ids [Hkv, N, min(topk, nblk)] int32 from the compressed-attention probabilities."""
+    _require_cuda(q, ck, lse, cu_q, cu_k)
+    lib = _lib.load()
+    n, hq, d = q.shape
+    hkv = ck.shape[1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    nblk = (int(max_seqlen_q) + block_size - 1) // block_size
+    t_out = min(topk, nblk)
+    dev = q.device
+    idx = torch.empty((hkv, n, t_out), dtype=torch.int32, device=dev)
+    bscore = torch.empty((hkv, n, nblk), dtype=torch.float32, device=dev) if return_block_score else None
+    ws_bytes = lib.fsa_cmp_topk_workspace_bytes(n, hkv, max(1, int(max_seqlen_k)))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    lse = lse.contiguous()
+    rc = lib.fsa_cmp_topk(_ptr(q), _ptr(ck), _ptr(lse), _DTYPE[q.dtype], q.stride(0), q.stride(1),
+                          ck.stride(0), ck.stride(1), _ptr(cu_q), _ptr(cu_k), cu_q.numel() - 1, n,
+                          int(max_seqlen_q), max(1, int(max_seqlen_k)), hq, hkv, d, kernel_size, kernel_stride,
+                          block_size, topk, init_blocks, local_blocks, 1 if scores_to_bf16 else 0,
+                          float(softmax_scale), _ptr(idx), _ptr(bscore), _ptr(ws), ws_bytes, _stream(dev))
+    _lib.check(rc, "fsa_cmp_topk")
+    return (idx, bscore) if return_block_score else idx

@@ -142,6 +142,64 @@ int fsa_selattn_bwd(const void* q, const void* k, const void* v, const void* o, 
                     void* dq, void* dk, void* dv /* contiguous [N,H,D] */,
                     void* workspace, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Compressed attention: every query against the compressed keys / values of
+ * its sequence; compressed key j is visible to the query at sequence-local
+ * position i iff i >= j*kernel_stride + kernel_size - 1.  Queries without a
+ * visible key get O = 0, LSE = -inf.
+ * Replaces CompressedAttention / _compressed_attention_fwd / _bwd and their
+ * kernels (nsa_ref/ops/compressed_attention.py:27-518, 521-829).
+ * ck / cv are [total_k, Hkv, D] with cu_seqlens_k [batch+1]; lse is [Hq, total_q]
+ * fp32 base 2; dq is contiguous [total_q, Hq, D], dck / dcv contiguous
+ * [total_k, Hkv, D].  max_seqlen_q is any upper bound of the longest sequence.
+ * ---------------------------------------------------------------------- */
+int fsa_cmpattn_fwd(const void* q, const void* ck, const void* cv, int32_t dtype,
+                    int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                    int64_t v_stride_n, int64_t v_stride_h,
+                    const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int32_t batch,
+                    int64_t total_q, int64_t max_seqlen_q, int32_t num_q_heads, int32_t num_kv_heads,
+                    int32_t head_dim, int32_t kernel_size, int32_t kernel_stride, float softmax_scale,
+                    void* o, int64_t o_stride_n, int64_t o_stride_h, float* lse, void* stream);
+
+size_t fsa_cmpattn_bwd_workspace_bytes(int64_t total_q, int64_t total_k, int64_t max_seqlen_q,
+                                       int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                       int32_t head_dim);
+
+int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, const void* o, const void* d_o,
+                    const float* lse, int32_t dtype,
+                    int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                    int64_t v_stride_n, int64_t v_stride_h, int64_t o_stride_n, int64_t o_stride_h,
+                    int64_t do_stride_n, int64_t do_stride_h,
+                    const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int32_t batch,
+                    int64_t total_q, int64_t total_k, int64_t max_seqlen_q,
+                    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                    int32_t kernel_size, int32_t kernel_stride, float softmax_scale,
+                    void* dq, void* dck, void* dcv, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Top-k block selection from the compressed-attention probabilities.
+ * Replaces _get_attention_score / score_kernel, transform_score /
+ * _transform_score_kernel and the torch.topk + sort + mask of
+ * nsa_ref/ops/compressed_attention.py:832-1003, 1006-1158, 1272-1315
+ * (per kv head, probabilities of the FIRST q head of the group).
+ *   topk_idx    [Hkv, total_q, min(topk, nblk)] int32 out, nblk = ceil(max_seqlen_q / block_size)
+ *   block_score [Hkv, total_q, nblk] fp32 out, optional (NULL to skip)
+ * scores_to_bf16 != 0 rounds the block scores to bf16 before the selection, as
+ * the reference's per-head path does.  Equal scores are ordered by lower block id.
+ * The workspace holds the fp32 probabilities.
+ * ---------------------------------------------------------------------- */
+size_t fsa_cmp_topk_workspace_bytes(int64_t total_q, int32_t num_kv_heads, int64_t max_seqlen_k);
+
+int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
+                 int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                 const int32_t* cu_seqlens_q, const int32_t* cu_seqlens_k, int32_t batch,
+                 int64_t total_q, int64_t max_seqlen_q, int64_t max_seqlen_k,
+                 int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                 int32_t kernel_size, int32_t kernel_stride, int32_t block_size, int32_t topk,
+                 int32_t init_blocks, int32_t local_blocks, int32_t scores_to_bf16, float softmax_scale,
+                 int32_t* topk_idx, float* block_score, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -101,7 +101,8 @@ def selected_attention_ref(
 
 
 def selected_attention_grads_ref(q, k, v, topk_idx, block_size, cu_seqlens, do, softmax_scale=None,
-                                 dtype=torch.float32, q_chunk: int = 128):
+                                 dtype=torch.float32, q_chunk: int = 128, round_dtype=None,
+                                 o_in=None, lse_in=None):
     """(O, LSE2, dQ, dK, dV) by the explicit backward formulas, chunk by chunk.
 
     FSA_topk_sparse_attention.py:1229-1237 and :1697-1709 with P = 2^(s - LSE2):
@@ -110,7 +111,20 @@ def selected_attention_grads_ref(q, k, v, topk_idx, block_size, cu_seqlens, do, 
     (dK/dV head sum: :1854-1855).  No autograd, so memory stays bounded; the
     formulas themselves are checked against autograd of the dense formulation
     and finite differences in the tests.
+
+    o_in / lse_in: the backward operator of the reference takes the saved forward
+    output and LSE as INPUTS (FSA_topk_sparse_attention.py:1715-1730: delta is
+    computed from the stored, dtype-rounded O and P from the stored LSE); when
+    given they are used in place of the recomputed ones, which is the functional
+    specification of the backward op.
+
+    round_dtype (bf16 / fp16) reproduces the reference kernels' rounding points:
+    P is cast to the input dtype before P^T dO and dS before dS K and dS^T Q
+    (FSA_topk_sparse_attention.py:1236, 1705-1706); accumulation stays in `dtype`.
     """
+    def rnd(x):
+        return x if round_dtype is None else x.to(round_dtype).to(dtype)
+
     N, Hq, D = q.shape
     Hkv = k.shape[1]
     g = Hq // Hkv
@@ -153,17 +167,20 @@ def selected_attention_grads_ref(q, k, v, topk_idx, block_size, cu_seqlens, do, 
                 s = torch.bmm(qc[:, kh], kg.transpose(1, 2)) * c
                 s = s.masked_fill(~valid[kh][:, None, :], float("-inf"))
                 lse = torch.logsumexp(s * (1.0 / LOG2E), dim=-1, keepdim=True) * LOG2E  # base 2
-                p = torch.exp2(s - lse)
-                o = torch.bmm(p, vg)
-                dp = torch.bmm(doc[:, kh], vg.transpose(1, 2))
-                delta = (o * doc[:, kh]).sum(-1, keepdim=True)
-                ds = softmax_scale * p * (dp - delta)
                 hs = slice(kh * g, (kh + 1) * g)
+                o = torch.bmm(torch.exp2(s - lse), vg)
+                lse_use = lse if lse_in is None else lse_in[hs, s0 + i0 : s0 + i1].to(dtype).t()[:, :, None]
+                o_use = o if o_in is None else o_in[s0 + i0 : s0 + i1, hs].to(dtype)
+                p = torch.exp2(s - lse_use)
+                dp = torch.bmm(doc[:, kh], vg.transpose(1, 2))
+                delta = (o_use * doc[:, kh]).sum(-1, keepdim=True)
+                ds = softmax_scale * p * (dp - delta)
                 o_out[s0 + i0 : s0 + i1, hs] = o
                 lse_out[hs, s0 + i0 : s0 + i1] = lse.squeeze(-1).t()
-                dq[s0 + i0 : s0 + i1, hs] = torch.bmm(ds, kg)
-                dkb[kh].index_add_(0, bsel[kh], torch.bmm(ds.transpose(1, 2), qc[:, kh]).reshape(C * T, B * D))
-                dvb[kh].index_add_(0, bsel[kh], torch.bmm(p.transpose(1, 2), doc[:, kh]).reshape(C * T, B * D))
+                ds_c, p_c = rnd(ds), rnd(p)
+                dq[s0 + i0 : s0 + i1, hs] = torch.bmm(ds_c, kg)
+                dkb[kh].index_add_(0, bsel[kh], torch.bmm(ds_c.transpose(1, 2), qc[:, kh]).reshape(C * T, B * D))
+                dvb[kh].index_add_(0, bsel[kh], torch.bmm(p_c.transpose(1, 2), doc[:, kh]).reshape(C * T, B * D))
         dk[s0:s1] = dkb.reshape(Hkv, nblk * B, D)[:, :L].permute(1, 0, 2)
         dv[s0:s1] = dvb.reshape(Hkv, nblk * B, D)[:, :L].permute(1, 0, 2)
     return o_out, lse_out, dq, dk, dv

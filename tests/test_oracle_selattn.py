@@ -103,6 +103,10 @@ def test_grads_match_dense_autograd_and_finite_differences():
     (og * do).sum().backward()
     assert torch.allclose(dq, qg.grad, atol=1e-11) and torch.allclose(dk, kg.grad, atol=1e-11)
     assert torch.allclose(dv, vg.grad, atol=1e-11) and torch.allclose(lse, lseg, atol=1e-11)
+    # rounding points switched on with an identity rounding change nothing
+    _, _, dq3, dk3, dv3 = orc.selected_attention_grads_ref(q, k, v, topk, 8, cu, do, dtype=torch.float64,
+                                                           round_dtype=torch.float64)
+    assert torch.equal(dq3, dq) and torch.equal(dk3, dk) and torch.equal(dv3, dv)
 
     def loss(q_, k_, v_):
         return float((orc.selected_attention_ref(q_, k_, v_, topk, 8, cu, dtype=torch.float64)[0] * do).sum())

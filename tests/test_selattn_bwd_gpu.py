@@ -6,7 +6,10 @@ blocks reach magnitudes where one unit in the last place of bf16 already exceeds
 2e-2 (ulp(4.0) = 0.031), so the bound applied per element is
     |got - ref| <= atol + ulp_rel * |ref|,   ulp_rel = 2^-8 (bf16) or 2^-11 (fp16),
 i.e. the stated max-abs tolerance plus the representability of the output dtype.
-The plain max-abs error is printed next to it.
+The plain max-abs error is printed next to it.  The backward is checked as the
+operator it is - (q, k, v, o, do, lse) -> (dq, dk, dv), the stored forward
+output and LSE being inputs as in the reference's own backward test - with the
+reference kernels' rounding points (P and dS cast to the input dtype).
 """
 import pytest
 import torch
@@ -47,7 +50,8 @@ def test_bwd_matches_oracle(dev, cu, hq, hkv, d, bk, t, dtype, std):
     dq, dk, dv = ops.selattn_bwd(qd, kd, vd, o, dod, lse, index)
     torch.cuda.synchronize()
     _, _, dq_r, dk_r, dv_r = orc.selected_attention_grads_ref(q.float(), k.float(), v.float(), topk, bk, cu,
-                                                              do.float())
+                                                              do.float(), round_dtype=dtype,
+                                                              o_in=o.float().cpu(), lse_in=lse.cpu())
     for name, got, ref in (("dq", dq, dq_r), ("dk", dk, dk_r), ("dv", dv, dv_r)):
         got = got.float().cpu()
         assert torch.isfinite(got).all(), name
