@@ -1,0 +1,429 @@
+// One-step decode for gfx950: one new query per request against its caches.
+//
+//   decode_attn_kernel (compressed mode): the g heads of a kv group attend every
+//       visible compressed key of the request; the raw scores of one "scoring"
+//       head are kept for the block selection.
+//   decode_attn_kernel (selected mode): the g heads attend the cached keys of
+//       the T selected blocks.
+//   decode_topk_kernel: probabilities -> re-binned block scores -> top-k ids.
+//
+// Both attention modes are HBM-bound streams of K/V rows (g rows of queries
+// only), so one work-group per (request, kv head) lets its four waves take
+// 64-key tiles round-robin: K fragments go straight from global memory into
+// MFMA operands, the V tile is staged in a wave-private LDS region and read
+// back transposed, and the waves' partial (m, l, O) are merged through LDS.
+// The query heads occupy the first g of the 32 MFMA columns; column g carries
+// the scoring head.
+//
+// Semantics: fsa_preview/ops/compressed_attention_decode.py:361-490 (attention),
+// :494-592 (scores), :284-357 (transform), :203-205 (top-k);
+// fsa_preview/ops/selected_attention_decode.py:8-42.
+#include "fsa_common.h"
+
+namespace fsa {
+
+constexpr int DEC_MODE_COMPRESSED = 0;
+constexpr int DEC_MODE_SELECTED = 1;
+constexpr int DEC_TILE = 64;
+
+struct DecParams {
+  const void* q;   // [B, Hq, D]
+  const void* k;   // [total, Hkv, D]
+  const void* v;
+  int64_t q_sb, q_sh, k_sn, k_sh, v_sn, v_sh;
+  const int32_t* cu_k;      // [B+1] rows of k / v per request
+  const int32_t* pos;       // compressed mode: position of the query
+  const int32_t* topk_idx;  // selected mode: [Hkv, B, T]
+  int batch, hq, hkv, g, topk, block_size, kernel_size, kernel_stride;
+  float scale_log2;
+  void* o;                  // [B, Hq, D] contiguous
+  float* lse;               // [Hq, B]
+  float* raw_score;         // compressed mode, optional: [Hkv, B, raw_ld] unscaled q.k of the scoring head
+  int64_t raw_ld;
+  int score_head_as_written;  // 0: first head of the group, 1: q-head with the kv head's own index
+};
+
+template <int D> struct DecLds {
+  static constexpr int VS = D + 16;
+  static constexpr int WAVE_BYTES = DEC_TILE * VS * 2;
+  static constexpr int MERGE_BYTES = 4 * ((D / 32) * 16 + 2) * 64 * 4;
+  static constexpr int BYTES = 4 * WAVE_BYTES > MERGE_BYTES ? 4 * WAVE_BYTES : MERGE_BYTES;
+};
+
+template <typename T, int D, int MODE>
+__global__ void __launch_bounds__(256)
+decode_attn_kernel(DecParams p) {
+  typedef typename Elem<T>::vec8 vec8;
+  typedef typename Elem<T>::vec4 vec4;
+  constexpr int VS = DecLds<D>::VS;
+  constexpr int NA = DEC_TILE / 32, NKS = D / 16, NDT = D / 32, NJ = DEC_TILE / 16;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int col = lane & 31, hh = lane >> 5;
+  T* Vs = reinterpret_cast<T*>(smem) + wv * (DEC_TILE * VS);
+
+  const int k0 = p.cu_k[b], len = p.cu_k[b + 1] - k0;
+  int n_tiles, n_keys = 0, tpb = 1;
+  if (MODE == DEC_MODE_COMPRESSED) {
+    const int qp = p.pos[b];
+    n_keys = qp >= p.kernel_size - 1 ? min(len, (qp - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
+    n_tiles = (n_keys + DEC_TILE - 1) / DEC_TILE;
+  } else {
+    tpb = (p.block_size + DEC_TILE - 1) / DEC_TILE;
+    n_tiles = p.topk * tpb;
+  }
+  const int32_t* sel = MODE == DEC_MODE_SELECTED ? p.topk_idx + ((int64_t)h * p.batch + b) * p.topk : nullptr;
+
+  // B operand: columns 0..g-1 = heads of the group, column g = scoring head (compressed mode)
+  vec8 qreg[NKS];
+  {
+    int hq_i = -1;
+    if (col < p.g) hq_i = h * p.g + col;
+    else if (MODE == DEC_MODE_COMPRESSED && col == p.g) hq_i = p.score_head_as_written ? h : h * p.g;
+    const T* qrow = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)max(hq_i, 0) * p.q_sh + hh * (D / 2);
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) qreg[ks] = hq_i >= 0 ? load16<vec8>(qrow + ks * 8) : zero8<T>();
+  }
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh + hh * (D / 2);
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
+  const T* vtr = Vs + (4 * hh + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
+  float m = -INFINITY, l = 0.f;
+  f32x16 oacc[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+
+  for (int tt = wv; tt < n_tiles; tt += 4) {
+    int row0, n_valid;
+    if (MODE == DEC_MODE_COMPRESSED) {
+      row0 = tt * DEC_TILE;
+      n_valid = min(DEC_TILE, n_keys - row0);
+    } else {
+      const int t = tt / tpb, sub = tt - t * tpb;
+      const int blk = sel[t];
+      bool dup = false;
+      for (int u = 0; u < t; ++u) dup |= sel[u] == blk;
+      row0 = blk * p.block_size + sub * DEC_TILE;
+      n_valid = (blk < 0 || dup) ? 0 : min(min(DEC_TILE, p.block_size - sub * DEC_TILE), len - row0);
+    }
+    if (n_valid <= 0) continue;  // uniform per wave
+    // K fragments straight from global memory
+    f32x16 acc[NA];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+      const int key = a * 32 + col;
+      const T* krow = kbase + (int64_t)(k0 + row0 + key) * p.k_sn;
+      vec8 kf[NKS];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) kf[ks] = key < n_valid ? load16<vec8>(krow + ks * 8) : zero8<T>();
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) acc[a] = Elem<T>::mfma32(kf[ks], qreg[ks], acc[a]);
+    }
+    // V tile -> wave-private LDS (rows past n_valid are zero so that 0 * garbage cannot appear)
+    for (int c = lane; c < DEC_TILE * (D / 8); c += 64) {
+      const int row = c / (D / 8), cc = c % (D / 8);
+      vec8 x = zero8<T>();
+      if (row < n_valid) x = load16<vec8>(vbase + (int64_t)(k0 + row0 + row) * p.v_sn + cc * 8);
+      store16(&Vs[row * VS + cc * 8], x);
+    }
+    if (MODE == DEC_MODE_COMPRESSED && p.raw_score && col == p.g) {
+      float* rs = p.raw_score + ((int64_t)h * p.batch + b) * p.raw_ld + row0;
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const int key0 = a * 32 + 8 * qd + 4 * hh;
+          if (row0 + key0 < p.raw_ld) {
+            f32x4 x;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = acc[a][4 * qd + e];
+            *reinterpret_cast<f32x4*>(rs + key0) = x;
+          }
+        }
+    }
+    float mx = m;
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+        const float sv = key < n_valid ? acc[a][i] : -INFINITY;
+        acc[a][i] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = fmaxf(mx, xor32(mx));
+    const float mref = mx * p.scale_log2;  // n_valid > 0, so mx is finite
+    const float alpha = exp2f(m * p.scale_log2 - mref);
+    float lsum = 0.f;
+    vec8 pk[NJ];
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pv = exp2f(acc[a][i] * p.scale_log2 - mref);
+        lsum += pv;
+        pk[a * 2 + (i >> 3)][i & 7] = (T)pv;
+      }
+    lsum += xor32(lsum);
+    l = l * alpha + lsum;
+    m = mx;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+#pragma unroll
+      for (int j = 0; j < NJ; ++j) {
+        vec8 vf = lds_read_tr8<T>(vtr + 16 * j * VS + dt * 32, 8 * VS);
+        oacc[dt] = Elem<T>::mfma32(vf, pk[j], oacc[dt]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // merge the four waves' partial results: lane-wise, the accumulator layout is the same in every wave
+  __syncthreads();
+  float* mg = reinterpret_cast<float*>(smem);
+  constexpr int PER = NDT * 16 + 2;
+  float* mine = mg + (wv * PER) * 64 + lane;
+  mine[0] = m;
+  mine[64] = l;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mine[(2 + dt * 16 + i) * 64] = oacc[dt][i];
+  __syncthreads();
+  if (wv != 0 || col >= p.g) return;
+  float mt = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) mt = fmaxf(mt, mg[(w * PER) * 64 + lane]);
+  float lt = 0.f, wgt[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float mw = mg[(w * PER) * 64 + lane];
+    wgt[w] = mw == -INFINITY ? 0.f : exp2f((mw - mt) * p.scale_log2);
+    lt += wgt[w] * mg[(w * PER + 1) * 64 + lane];
+  }
+  const float inv_l = lt > 0.f ? 1.f / lt : 0.f;
+  const int hq_i = h * p.g + col;
+  T* orow = reinterpret_cast<T*>(p.o) + ((int64_t)b * p.hq + hq_i) * D + 4 * hh;
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      vec4 x;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float s = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) s += wgt[w] * mg[(w * PER + 2 + dt * 16 + 4 * qd + e) * 64 + lane];
+        x[e] = (T)(s * inv_l);
+      }
+      store8(orow + dt * 32 + 8 * qd, x);
+    }
+  if (hh == 0) p.lse[(int64_t)hq_i * p.batch + b] = lt > 0.f ? mt * p.scale_log2 + log2f(lt) : -INFINITY;
+}
+
+// ------------------------------------------------------------------ top-k ----
+struct DecTopkParams {
+  const float* raw_score;  // [Hkv, B, raw_ld]
+  int64_t raw_ld;
+  const float* lse;        // [Hq, B]
+  const int32_t* cu_ck;    // [B+1] compressed rows per request
+  const int32_t* pos;      // [B]
+  const int32_t* seqlens;  // [B] cache length including the new token
+  int batch, hkv, g;
+  int kernel_size, kernel_stride, block_size, topk, init_blocks, local_blocks;
+  int as_written;
+  float scale_log2;
+  int32_t* topk_idx;       // [Hkv, B, topk]
+  float* block_score;      // optional [Hkv, B, score_ld]
+  int64_t score_ld;
+};
+
+// one wave per (request, kv head)
+__global__ void __launch_bounds__(64)
+decode_topk_kernel(DecTopkParams p) {
+  extern __shared__ float bs[];
+  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int nc = p.cu_ck[b + 1] - p.cu_ck[b];
+  const int qp = p.pos[b];
+  const int n_vis = qp >= p.kernel_size - 1 ? min(nc, (qp - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
+  const int len = p.seqlens[b];
+  const int nblk = p.as_written ? (nc + p.block_size - 1) / p.block_size : (len + p.block_size - 1) / p.block_size;
+  const int bq = p.as_written ? 0 : (len - 1) / p.block_size;
+  const int hq_s = p.as_written ? h : h * p.g;
+  const float lse_r = p.lse[(int64_t)hq_s * p.batch + b];
+  const int na = p.kernel_size / p.kernel_stride, ne = p.block_size / p.kernel_stride;
+  const int n_off = na + ne - 1, pad = na - 1;
+  const float* rs = p.raw_score + ((int64_t)h * p.batch + b) * p.raw_ld;
+  for (int blk = lane; blk < nblk; blk += 64) {
+    float acc = 0.f;
+    const int c0 = blk * ne - pad;
+    for (int o = 0; o < n_off; ++o) {
+      const int c = c0 + o;
+      if (c >= 0 && c < n_vis) {
+        const int wgt = min(min(o, n_off - 1 - o), min(na, ne) - 1) + 1;
+        acc += (float)wgt * exp2f(rs[c] * p.scale_log2 - lse_r);
+      }
+    }
+    if (blk < p.init_blocks || (bq >= blk && bq < blk + p.local_blocks)) acc = INFINITY;
+    bs[blk] = acc;
+    if (p.block_score) p.block_score[((int64_t)h * p.batch + b) * p.score_ld + blk] = acc;
+  }
+  if (p.block_score)
+    for (int64_t blk = nblk + lane; blk < p.score_ld; blk += 64)
+      p.block_score[((int64_t)h * p.batch + b) * p.score_ld + blk] = -INFINITY;
+  __builtin_amdgcn_wave_barrier();
+  int32_t* out = p.topk_idx + ((int64_t)h * p.batch + b) * p.topk;
+  for (int t = 0; t < p.topk; ++t) {
+    float best = -2.f;
+    int best_id = 0x7fffffff;
+    for (int blk = lane; blk < nblk; blk += 64) {
+      const float vv = bs[blk];
+      if (vv > best) {
+        best = vv;
+        best_id = blk;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(best_id, o, 64);
+      if (ov > best || (ov == best && oi < best_id)) {
+        best = ov;
+        best_id = oi;
+      }
+    }
+    if (lane == 0) {
+      out[t] = best >= 0.f ? best_id : -1;  // fewer than topk blocks exist
+      if (best >= 0.f) bs[best_id] = -1.f;
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+template <typename T, int D, int MODE>
+static int dec_launch(const DecParams& p, hipStream_t stream) {
+  constexpr int lds = DecLds<D>::BYTES;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)decode_attn_kernel<T, D, MODE>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(%d B LDS): %s", lds, hipGetErrorString(e));
+      return (int)e;
+    }
+  }
+  ProfScope ps_(MODE == DEC_MODE_COMPRESSED ? "decode_cmpattn" : "decode_selattn", stream);
+  decode_attn_kernel<T, D, MODE><<<dim3(p.batch, p.hkv), 256, lds, stream>>>(p);
+  return 0;
+}
+
+template <int MODE>
+static int dec_dispatch(int dtype, int head_dim, const DecParams& p, hipStream_t stream) {
+  if (dtype == FSA_BF16) {
+    if (head_dim == 64) return dec_launch<__bf16, 64, MODE>(p, stream);
+    if (head_dim == 128) return dec_launch<__bf16, 128, MODE>(p, stream);
+    if (head_dim == 256) return dec_launch<__bf16, 256, MODE>(p, stream);
+  } else {
+    if (head_dim == 64) return dec_launch<_Float16, 64, MODE>(p, stream);
+    if (head_dim == 128) return dec_launch<_Float16, 128, MODE>(p, stream);
+    if (head_dim == 256) return dec_launch<_Float16, 256, MODE>(p, stream);
+  }
+  set_error("decode: head_dim=%d not supported (64, 128, 256)", head_dim);
+  return FSA_ERR_UNSUPPORTED;
+}
+
+}  // namespace fsa
+
+using namespace fsa;
+
+extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv, int32_t dtype,
+                                  int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n,
+                                  int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                                  const int32_t* cu_ck, const int32_t* pos, int32_t batch,
+                                  int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                  int32_t kernel_size, int32_t kernel_stride, float softmax_scale,
+                                  int32_t score_head_as_written, void* o, float* lse, float* raw_score,
+                                  int64_t raw_ld, void* stream_) {
+  FSA_CHECK_ARG(q && ck && cv && cu_ck && pos && o && lse, "fsa_decode_cmpattn: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_decode_cmpattn: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
+                "fsa_decode_cmpattn: num_q_heads must be a multiple of num_kv_heads");
+  const int g = num_q_heads / num_kv_heads;
+  FSA_CHECK_ARG(g <= 31, "fsa_decode_cmpattn: at most 31 query heads per kv head");
+  FSA_CHECK_ARG(batch >= 1 && kernel_size >= 1 && kernel_stride >= 1, "fsa_decode_cmpattn: bad sizes");
+  FSA_CHECK_ARG(!raw_score || (raw_ld >= 4 && raw_ld % 4 == 0), "fsa_decode_cmpattn: raw_ld must be a multiple of 4");
+  FSA_CHECK_ARG(!score_head_as_written || num_kv_heads <= num_q_heads, "fsa_decode_cmpattn: bad scoring head");
+  DecParams p = {};
+  p.q = q; p.k = ck; p.v = cv; p.q_sb = q_stride_b; p.q_sh = q_stride_h;
+  p.k_sn = k_stride_n; p.k_sh = k_stride_h; p.v_sn = v_stride_n; p.v_sh = v_stride_h;
+  p.cu_k = cu_ck; p.pos = pos; p.batch = batch; p.hq = num_q_heads; p.hkv = num_kv_heads; p.g = g;
+  p.kernel_size = kernel_size; p.kernel_stride = kernel_stride; p.scale_log2 = softmax_scale * LOG2E;
+  p.o = o; p.lse = lse; p.raw_score = raw_score; p.raw_ld = raw_ld;
+  p.score_head_as_written = score_head_as_written;
+  int rc = dec_dispatch<DEC_MODE_COMPRESSED>(dtype, head_dim, p, (hipStream_t)stream_);
+  if (rc) return rc;
+  FSA_CHECK_LAUNCH("fsa_decode_cmpattn");
+  return 0;
+}
+
+extern "C" int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const float* lse,
+                               const int32_t* cu_ck, const int32_t* pos, const int32_t* seqlens,
+                               int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                               int32_t kernel_size, int32_t kernel_stride, int32_t block_size,
+                               int32_t topk, int32_t init_blocks, int32_t local_blocks,
+                               int32_t as_written, float softmax_scale, int64_t max_blocks,
+                               int32_t* topk_idx, float* block_score, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FSA_CHECK_ARG(raw_score && lse && cu_ck && pos && seqlens && topk_idx, "fsa_decode_topk: null pointer");
+  FSA_CHECK_ARG(batch >= 1 && topk >= 1 && num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
+                "fsa_decode_topk: bad sizes");
+  FSA_CHECK_ARG(kernel_stride >= 1 && kernel_size % kernel_stride == 0 && block_size % kernel_stride == 0,
+                "fsa_decode_topk: kernel_size and block_size must be multiples of kernel_stride");
+  FSA_CHECK_ARG(max_blocks >= 1 && max_blocks * 4 <= 64 * 1024,
+                "fsa_decode_topk: max_blocks must be in [1, 16384]");
+  DecTopkParams p = {};
+  p.raw_score = raw_score; p.raw_ld = raw_ld; p.lse = lse; p.cu_ck = cu_ck; p.pos = pos; p.seqlens = seqlens;
+  p.batch = batch; p.hkv = num_kv_heads; p.g = num_q_heads / num_kv_heads;
+  p.kernel_size = kernel_size; p.kernel_stride = kernel_stride; p.block_size = block_size; p.topk = topk;
+  p.init_blocks = init_blocks; p.local_blocks = local_blocks; p.as_written = as_written;
+  p.scale_log2 = softmax_scale * LOG2E; p.topk_idx = topk_idx; p.block_score = block_score;
+  p.score_ld = max_blocks;
+  {
+    ProfScope ps_("decode_topk", stream);
+    decode_topk_kernel<<<dim3(batch, num_kv_heads), 64, (size_t)max_blocks * 4, stream>>>(p);
+  }
+  FSA_CHECK_LAUNCH("fsa_decode_topk");
+  return 0;
+}
+
+extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
+                                  int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n,
+                                  int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                                  const int32_t* cu_k, const int32_t* topk_idx, int32_t batch,
+                                  int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                  int32_t topk, int32_t block_size, float softmax_scale, void* o,
+                                  float* lse, void* stream_) {
+  FSA_CHECK_ARG(q && k_cache && v_cache && cu_k && topk_idx && o && lse, "fsa_decode_selattn: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_decode_selattn: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
+                "fsa_decode_selattn: num_q_heads must be a multiple of num_kv_heads");
+  FSA_CHECK_ARG(num_q_heads / num_kv_heads <= 32, "fsa_decode_selattn: at most 32 query heads per kv head");
+  FSA_CHECK_ARG(batch >= 1 && topk >= 1 && block_size >= 1, "fsa_decode_selattn: bad sizes");
+  DecParams p = {};
+  p.q = q; p.k = k_cache; p.v = v_cache; p.q_sb = q_stride_b; p.q_sh = q_stride_h;
+  p.k_sn = k_stride_n; p.k_sh = k_stride_h; p.v_sn = v_stride_n; p.v_sh = v_stride_h;
+  p.cu_k = cu_k; p.topk_idx = topk_idx; p.batch = batch; p.hq = num_q_heads; p.hkv = num_kv_heads;
+  p.g = num_q_heads / num_kv_heads; p.topk = topk; p.block_size = block_size;
+  p.scale_log2 = softmax_scale * LOG2E; p.o = o; p.lse = lse;
+  int rc = dec_dispatch<DEC_MODE_SELECTED>(dtype, head_dim, p, (hipStream_t)stream_);
+  if (rc) return rc;
+  FSA_CHECK_LAUNCH("fsa_decode_selattn");
+  return 0;
+}

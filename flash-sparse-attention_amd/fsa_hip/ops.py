@@ -229,3 +229,73 @@ def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_
                           float(softmax_scale), _ptr(idx), _ptr(bscore), _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_cmp_topk")
     return (idx, bscore) if return_block_score else idx
+
+
+def decode_cmpattn(q, ck, cv, cu_ck, pos, kernel_size, kernel_stride, max_ck, softmax_scale=None,
+                   want_scores=True, score_head_as_written=False):
+    """Decode-step compressed attention for a batch of requests.
+
+    q [B,Hq,D]; ck/cv [total_ck,Hkv,D] with cu_ck [B+1]; pos [B] int32 query positions;
+    max_ck: host upper bound of the longest compressed cache.
+    Returns (o [B,Hq,D], lse [Hq,B], raw_score [Hkv,B,ld] or None)."""
+    _require_cuda(q, ck, cv, cu_ck, pos)
+    assert q.dtype in _DTYPE and q.dtype == ck.dtype == cv.dtype
+    assert q.dim() == 3 and q.stride(2) == 1 and ck.stride(2) == 1 and cv.stride(2) == 1
+    lib = _lib.load()
+    b, hq, d = q.shape
+    hkv = ck.shape[1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    dev = q.device
+    o = torch.empty((b, hq, d), dtype=q.dtype, device=dev)
+    lse = torch.empty((hq, b), dtype=torch.float32, device=dev)
+    ld = (max(int(max_ck), 1) + 3) // 4 * 4
+    raw = torch.empty((hkv, b, ld), dtype=torch.float32, device=dev) if want_scores else None
+    rc = lib.fsa_decode_cmpattn(_ptr(q), _ptr(ck), _ptr(cv), _DTYPE[q.dtype], q.stride(0), q.stride(1),
+                                ck.stride(0), ck.stride(1), cv.stride(0), cv.stride(1), _ptr(cu_ck), _ptr(pos),
+                                b, hq, hkv, d, kernel_size, kernel_stride, float(softmax_scale),
+                                1 if score_head_as_written else 0, _ptr(o), _ptr(lse), _ptr(raw), ld,
+                                _stream(dev))
+    _lib.check(rc, "fsa_decode_cmpattn")
+    return o, lse, raw
+
+
+def decode_topk(raw_score, lse, cu_ck, pos, seqlens, num_q_heads, kernel_size, kernel_stride, block_size,
+                topk, max_blocks, init_blocks=1, local_blocks=2, softmax_scale=1.0, as_written=False,
+                return_block_score=False):
+    """Top-k block ids [Hkv,B,topk] int32 (descending score) for the decode step."""
+    _require_cuda(raw_score, lse, cu_ck, pos, seqlens)
+    lib = _lib.load()
+    hkv, b, ld = raw_score.shape
+    dev = raw_score.device
+    idx = torch.empty((hkv, b, topk), dtype=torch.int32, device=dev)
+    bscore = torch.empty((hkv, b, max_blocks), dtype=torch.float32, device=dev) if return_block_score else None
+    rc = lib.fsa_decode_topk(_ptr(raw_score), ld, _ptr(lse), _ptr(cu_ck), _ptr(pos), _ptr(seqlens), b,
+                             num_q_heads, hkv, kernel_size, kernel_stride, block_size, topk, init_blocks,
+                             local_blocks, 1 if as_written else 0, float(softmax_scale), int(max_blocks),
+                             _ptr(idx), _ptr(bscore), _stream(dev))
+    _lib.check(rc, "fsa_decode_topk")
+    return (idx, bscore) if return_block_score else idx
+
+
+def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scale=None):
+    """Decode-step selected attention: (o [B,Hq,D], lse [Hq,B])."""
+    _require_cuda(q, k_cache, v_cache, cu_k, topk_idx)
+    assert q.dtype in _DTYPE and q.dtype == k_cache.dtype == v_cache.dtype
+    assert topk_idx.dtype == torch.int32 and topk_idx.is_contiguous()
+    assert q.stride(2) == 1 and k_cache.stride(2) == 1 and v_cache.stride(2) == 1
+    lib = _lib.load()
+    b, hq, d = q.shape
+    hkv = k_cache.shape[1]
+    assert topk_idx.shape[0] == hkv and topk_idx.shape[1] == b
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    dev = q.device
+    o = torch.empty((b, hq, d), dtype=q.dtype, device=dev)
+    lse = torch.empty((hq, b), dtype=torch.float32, device=dev)
+    rc = lib.fsa_decode_selattn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _DTYPE[q.dtype], q.stride(0), q.stride(1),
+                                k_cache.stride(0), k_cache.stride(1), v_cache.stride(0), v_cache.stride(1),
+                                _ptr(cu_k), _ptr(topk_idx), b, hq, hkv, d, topk_idx.shape[2], block_size,
+                                float(softmax_scale), _ptr(o), _ptr(lse), _stream(dev))
+    _lib.check(rc, "fsa_decode_selattn")
+    return o, lse

@@ -200,6 +200,54 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
                  int32_t* topk_idx, float* block_score, void* workspace, size_t workspace_bytes,
                  void* stream);
 
+/* ------------------------------------------------------------------------
+ * One-step decode: ONE new query per request, a batch of requests per call
+ * (the reference handles a batch of one).  q is [B, Hq, D]; caches are packed
+ * [total_rows, Hkv, D] with cu_* [B+1]; o is contiguous [B, Hq, D]; lse [Hq, B].
+ *
+ * fsa_decode_cmpattn replaces _compressed_attention_fwd_decode /
+ * forward_kernel_decode and the score recomputation of score_kernel_decode
+ * (fsa_preview/ops/compressed_attention_decode.py:15-97, 361-490, 494-592):
+ * compressed key j is visible iff j*stride + ks - 1 <= pos[b].  If raw_score is
+ * not NULL the unscaled q.k of the scoring head of every kv head is stored in
+ * raw_score[Hkv, B, raw_ld] (raw_ld >= longest visible compressed length,
+ * multiple of 4); the scoring head is the first head of the group, or - with
+ * score_head_as_written - the q head whose index equals the kv head's (:560,568).
+ *
+ * fsa_decode_topk replaces transform_score_decode + topk (:284-357, 203-205):
+ * ids ordered by descending score (equal scores by lower id), -1 where fewer
+ * than topk blocks exist.  as_written = 1 reproduces the reference literally
+ * (candidate blocks = ceil(compressed_len / block_size), own block taken as 0);
+ * as_written = 0 uses ceil(seqlens[b] / block_size) blocks and own block
+ * (seqlens[b]-1) / block_size.  block_score is optional [Hkv, B, max_blocks].
+ *
+ * fsa_decode_selattn replaces _topk_sparse_attention_decode
+ * (fsa_preview/ops/selected_attention_decode.py:8-42): the g heads of a group
+ * attend every cached key of the selected blocks (ids < 0, past the cache or
+ * repeated are ignored).
+ * ---------------------------------------------------------------------- */
+int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv, int32_t dtype,
+                       int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                       int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_ck, const int32_t* pos,
+                       int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                       int32_t kernel_size, int32_t kernel_stride, float softmax_scale,
+                       int32_t score_head_as_written, void* o, float* lse, float* raw_score,
+                       int64_t raw_ld, void* stream);
+
+int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const float* lse, const int32_t* cu_ck,
+                    const int32_t* pos, const int32_t* seqlens, int32_t batch, int32_t num_q_heads,
+                    int32_t num_kv_heads, int32_t kernel_size, int32_t kernel_stride, int32_t block_size,
+                    int32_t topk, int32_t init_blocks, int32_t local_blocks, int32_t as_written,
+                    float softmax_scale, int64_t max_blocks, int32_t* topk_idx, float* block_score,
+                    void* stream);
+
+int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
+                       int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                       int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_k,
+                       const int32_t* topk_idx, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                       int32_t head_dim, int32_t topk, int32_t block_size, float softmax_scale, void* o,
+                       float* lse, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
