@@ -1,0 +1,58 @@
+"""The C-ABI library loads without a GPU and exports every symbol include/fsa_hip.h declares;
+host-side argument checks of entry points that need no device work."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from fsa_hip import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "fsa_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fsa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    names = _declared()
+    assert len(names) >= 20
+    lib = _lib.load()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/fsa_hip.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes prototype"
+    assert set(_lib.SIGNATURES) <= set(names)
+
+
+def test_version_and_host_arithmetic():
+    lib = _lib.load()
+    assert lib.fsa_version() >= 100
+    # tiles upper bound: ceil(N*T*g / rows) + max_blocks
+    assert lib.fsa_max_tiles(65536, 16, 1, 1024, 1025) == 65536 * 16 // 1024 + 1025
+    assert lib.fsa_index_workspace_bytes(65536, 16, 4, 1025) >= 4 * 65536 * 16 * 4 * 4
+    a = lib.fsa_selattn_fwd_workspace_bytes(65536, 4, 4, 128, 16, 1025)
+    b = lib.fsa_selattn_fwd_workspace_bytes(65536, 16, 4, 128, 16, 1025)
+    assert b > 3 * a  # partial buffers scale with the GQA group
+
+
+def test_invalid_arguments_are_reported_not_launched():
+    lib = _lib.load()
+    rc = lib.fsa_build_tiles(None, 4, 10, 1, 128, None, None)
+    assert rc == -1 and b"null" in lib.fsa_last_error()
+    rc = lib.fsa_build_index(None, 0, 0, None, 1, 16, 1, 4, 64, 2, None, None, None, None, None, None, 0, None)
+    assert rc == -1
+    with pytest.raises(ValueError):
+        _lib.check(rc, "fsa_build_index")
+
+
+def test_wrappers_refuse_cpu_tensors():
+    import torch
+
+    from fsa_hip import ops
+
+    t = torch.zeros(1, 4, 2, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.build_index(t, torch.tensor([0, 4], dtype=torch.int32), 64)
