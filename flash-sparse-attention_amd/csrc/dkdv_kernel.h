@@ -87,11 +87,18 @@ template <int D, int BK> struct KvCfg {
   static constexpr int CPT = KV_R * CPR / NT;  // chunks per thread and tensor
   static constexpr int ROW_STEP = NT / CPR;
   static constexpr int BYTES = 2 * KV_R * QS * 2 + KV_R * 12;
+  // with the fused dQ: K of the block (natural layout) and the dS^T tile [BK][KV_R]
+  static constexpr int KS = D + 8;
+  static constexpr int DSS = KV_R + 8;
+  static constexpr int BYTES_FUSED = BYTES + (BK * KS + BK * DSS) * 2;
   static constexpr int MIN_WAVES = (D <= 128 && NT <= 256) ? 2 : 1;  // work-groups per CU the registers allow
   static_assert(KV_R * CPR % NT == 0, "tile must divide evenly over the threads");
 };
 
-template <typename T, int D, int BK, int MODE>
+// FUSE_DQ (selected mode): the work-group also produces the partial dQ rows of
+// its (query, block) pairs - dQ^T = K^T dS^T with dS^T exchanged between the
+// waves through LDS - so Q and dO are gathered once for dQ, dK and dV.
+template <typename T, int D, int BK, int MODE, bool FUSE_DQ = false>
 __global__ void __launch_bounds__((KvCfg<D, BK>::NT), (KvCfg<D, BK>::MIN_WAVES))
 attn_bwd_dkdv_kernel(SelBwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
@@ -104,6 +111,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   float* lse_s = reinterpret_cast<float*>(Os + KV_R * QS);
   float* del_s = lse_s + KV_R;
   int* lim_s = reinterpret_cast<int*>(del_s + KV_R);
+  T* Kl = reinterpret_cast<T*>(lim_s + KV_R);   // FUSE_DQ only
+  T* dSs = Kl + BK * C::KS;                     // FUSE_DQ only
 
   const int h = blockIdx.y;
   const int64_t nbp1 = p.max_blocks + 1;
@@ -141,6 +150,15 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     }
   }
 
+  if (FUSE_DQ) {
+    const T* kb = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
+    for (int c = tid; c < BK * (D / 8); c += C::NT) {
+      const int row = c / (D / 8), cc = c % (D / 8);
+      vec8 x = zero8<T>();
+      if (row < blk.n_keys_valid) x = load16<vec8>(kb + (int64_t)(blk.key_row0 + row) * p.k_sn + cc * 8);
+      store16(&Kl[row * C::KS + cc * 8], x);
+    }
+  }
   const int32_t* toks = MODE == KV_MODE_SELECTED ? p.sel_tokens + (int64_t)h * p.cap + start : nullptr;
   // row r of the block -> global query row
   auto row_token = [&](int r) {
@@ -256,6 +274,12 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         dsk[rt][i] = (T)ds;
       }
     }
+    if (FUSE_DQ) {
+      // dS^T[key][row] for the whole tile: every lane owns 4 consecutive rows of its key
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt) store8(&dSs[key * C::DSS + rt * 16 + 4 * kg], dsk[rt]);
+      __syncthreads();
+    }
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
       vec8 pb = __builtin_shufflevector(pk[2 * u], pk[2 * u + 1], 0, 1, 2, 3, 4, 5, 6, 7);
@@ -266,6 +290,37 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
         vec8 qa = lds_read_tr8<T>(&Qs[32 * u * QS + tr_off + 16 * t], 16 * QS);
         dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
+      }
+    }
+    if (FUSE_DQ) {
+      // dQ^T[d][row] = sum over the block's keys of K^T[d][key] dS^T[key][row]; row tiles are
+      // dealt round-robin to the waves, both operands come from transposing LDS reads
+      T* dqpart = reinterpret_cast<T*>(p.dq_part);
+      const int64_t prow0 = ((int64_t)h * p.cap + start) * p.g;
+      const int ktr_off = (4 * kg + (l16 >> 2)) * C::KS + 4 * (l16 & 3);   // + 32*u*KS + 16*t
+      const int str_off = (4 * kg + (l16 >> 2)) * C::DSS + 4 * (l16 & 3);  // + 32*u*DSS + 16*rt
+      for (int rt = wv; rt < NRT; rt += C::NW) {
+        vec8 dsb[BK / 32];
+#pragma unroll
+        for (int u = 0; u < BK / 32; ++u)
+          dsb[u] = lds_read_tr8<T>(&dSs[32 * u * C::DSS + str_off + 16 * rt], 16 * C::DSS);
+        const int r = base + rt * 16 + l16;
+        T* orow = dqpart + (prow0 + r) * D + 4 * kg;
+#pragma unroll
+        for (int t = 0; t < NDT; ++t) {
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int u = 0; u < BK / 32; ++u) {
+            vec8 ka = lds_read_tr8<T>(&Kl[32 * u * C::KS + ktr_off + 16 * t], 16 * C::KS);
+            acc = Elem<T>::mfma16(ka, dsb[u], acc);
+          }
+          if (r < row_hi) {
+            vec4 x;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) x[i] = (T)acc[i];
+            store8(orow + 16 * t, x);
+          }
+        }
       }
     }
     __syncthreads();

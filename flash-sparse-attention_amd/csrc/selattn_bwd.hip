@@ -21,6 +21,8 @@
 #include "fsa_common.h"
 #include "dkdv_kernel.h"
 
+#include <stdlib.h>
+
 namespace fsa {
 
 // ---------------------------------------------------------------- delta ----
@@ -181,7 +183,7 @@ selattn_bwd_dq_kernel(SelBwdParams p) {
 template <typename T, int D>
 __global__ void __launch_bounds__(256)
 selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __restrict__ slot_of,
-                             int64_t cap, int64_t n_tokens, int hq, int g, int topk,
+                             int64_t cap, int64_t n_tokens, int hq, int g, int topk, int natural,
                              T* __restrict__ dq /* contiguous [N, Hq, D] */) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
@@ -204,6 +206,13 @@ selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __res
     vec8 x = load16<vec8>(dq_part + prow * D + sub * 8);
 #pragma unroll
     for (int e = 0; e < 8; ++e) accv[e] += (float)x[e];
+  }
+  if (natural) {  // partial rows written by the fused kernel are in plain d order
+    vec8 out;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = (T)accv[e];
+    store16(dq + (tok * hq + hq_i) * D + sub * 8, out);
+    return;
   }
   const int pos = sub * 8;
   const int hh = pos / (D / 2), rem = pos % (D / 2);
@@ -240,6 +249,16 @@ static BwdWs bwd_ws_layout(int64_t n, int hq, int hkv, int d, int topk, int bk, 
   return w;
 }
 
+// FSA_BWD_SPLIT=1 selects the two-kernel backward (separate dQ and dK/dV kernels, each
+// gathering Q and dO); the default is the fused kernel.  Read once.
+static bool fused_dq() {
+  static const bool v = [] {
+    const char* e = getenv("FSA_BWD_SPLIT");
+    return !(e && e[0] == '1');
+  }();
+  return v;
+}
+
 template <typename K> static int set_lds(K kernel, int bytes) {
   if (bytes <= 48 * 1024) return 0;
   hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
@@ -253,17 +272,26 @@ template <typename K> static int set_lds(K kernel, int bytes) {
 template <typename T, int D, int BK>
 static int launch_bwd(const SelBwdParams& pdq, const SelBwdParams& pkv, int hkv, int64_t tiles_dq,
                       int64_t tiles_kv, hipStream_t stream) {
-  int rc = set_lds(selattn_bwd_dq_kernel<T, D, BK>, DqLds<D, BK>::BYTES);
-  if (rc) return rc;
-  rc = set_lds(attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED>, KvCfg<D, BK>::BYTES);
-  if (rc) return rc;
-  {
-    ProfScope ps_("selattn_bwd_dq", stream);
-    selattn_bwd_dq_kernel<T, D, BK><<<dim3((unsigned)tiles_dq, hkv), DQ_THREADS, DqLds<D, BK>::BYTES, stream>>>(pdq);
-  }
-  {
-    ProfScope ps_("selattn_bwd_dkdv", stream);
-    attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES, stream>>>(pkv);
+  int rc = 0;
+  if (fused_dq()) {
+    rc = set_lds(attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED, true>, KvCfg<D, BK>::BYTES_FUSED);
+    if (rc) return rc;
+    ProfScope ps_("selattn_bwd_dqdkdv", stream);
+    attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED, true>
+        <<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES_FUSED, stream>>>(pkv);
+  } else {
+    rc = set_lds(selattn_bwd_dq_kernel<T, D, BK>, DqLds<D, BK>::BYTES);
+    if (rc) return rc;
+    rc = set_lds(attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED>, KvCfg<D, BK>::BYTES);
+    if (rc) return rc;
+    {
+      ProfScope ps_("selattn_bwd_dq", stream);
+      selattn_bwd_dq_kernel<T, D, BK><<<dim3((unsigned)tiles_dq, hkv), DQ_THREADS, DqLds<D, BK>::BYTES, stream>>>(pdq);
+    }
+    {
+      ProfScope ps_("selattn_bwd_dkdv", stream);
+      attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES, stream>>>(pkv);
+    }
   }
   {
     ProfScope ps_("selattn_bwd_dkdv_reduce", stream);
@@ -309,7 +337,8 @@ static int launch_rowwise(int d, const void* o, int64_t o_sn, int64_t o_sh, cons
                                                                 delta);                            \
     else                                                                                           \
       selattn_bwd_dq_reduce_kernel<T, DD><<<grid, 256, 0, stream>>>((const T*)dq_part, slot_of, cap, \
-                                                                    n, hq, g, topk, (T*)dq);       \
+                                                                    n, hq, g, topk,                \
+                                                                    fused_dq() ? 1 : 0, (T*)dq);   \
     return 0;                                                                                      \
   }
   FSA_CASE(64)
