@@ -513,7 +513,7 @@ static CmpBwdWs cmp_bwd_ws(int64_t n, int64_t n_k, int64_t max_q, int batch, int
   const int g = hq / hkv;
   w.max_blocks = (n_k + CMP_BK - 1) / CMP_BK + batch;
   // a key tile is seen by at most max_q queries of its sequence; rows = queries * g
-  w.max_tiles = w.max_blocks * ((max_q * g + KV_TILE_ROWS - 1) / KV_TILE_ROWS + 1);
+  w.max_tiles = w.max_blocks * ((max_q * g + kv_tile_rows(g) - 1) / kv_tile_rows(g) + 1);
   w.off_delta = 0;
   w.off_cu_tiles = align_up((size_t)n * hq * 4, 256);
   w.off_counts = w.off_cu_tiles + align_up((size_t)(batch + 1) * 4, 256);
@@ -678,7 +678,7 @@ extern "C" int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, co
   int32_t* tile_prefix = (int32_t*)(wsp + ws.off_tiles);
   cmp_kv_blocks_kernel<<<1, 256, 0, stream>>>(cu_seqlens_q, cu_seqlens_k, batch, num_kv_heads, ws.max_blocks,
                                               kernel_size, kernel_stride, cu_tiles, counts);
-  rc = fsa_build_tiles(counts, num_kv_heads, ws.max_blocks, g, KV_TILE_ROWS, tile_prefix, stream_);
+  rc = fsa_build_tiles(counts, num_kv_heads, ws.max_blocks, g, kv_tile_rows(g), tile_prefix, stream_);
   if (rc) return rc;
 
   CmpParams p = {};
@@ -699,6 +699,7 @@ extern "C" int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, co
   kv.batch = batch; kv.max_blocks = ws.max_blocks; kv.cap = 0; kv.n_tokens = total_q; kv.g = g;
   kv.scale = softmax_scale; kv.scale_log2 = softmax_scale * LOG2E;
   kv.dq_part = nullptr; kv.dkdv_part = (float*)(wsp + ws.off_part); kv.max_tiles = ws.max_tiles;
+  kv.kv_tile_rows = kv_tile_rows(g);
   kv.dk = dck; kv.dv = dcv; kv.dk_sn = (int64_t)num_kv_heads * head_dim; kv.dk_sh = head_dim;
   kv.cu_seqlens_k = cu_seqlens_k; kv.kernel_size = kernel_size; kv.kernel_stride = kernel_stride;
 

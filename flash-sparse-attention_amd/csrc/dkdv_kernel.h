@@ -36,6 +36,7 @@ struct SelBwdParams {
   void* dq_part;     // [Hkv, cap, g, D] lane-native order
   float* dkdv_part;  // [Hkv, max_tiles, 2, BK, D]
   int64_t max_tiles;
+  int kv_tile_rows;  // rows per work-group of the dK/dV kernel
   void* dk;          // rows of k's shape, strides dk_sn / dk_sh
   void* dv;
   int64_t dk_sn, dk_sh;
@@ -77,12 +78,13 @@ template <int MODE, int BK> struct KvBlock {
 
 // ----------------------------------------------------------------- dkdv ----
 constexpr int KV_R = 64;             // gathered rows per pass
-constexpr int KV_TILE_ROWS = 4096;   // rows per work-group
+constexpr int KV_TILE_ROWS = 4096;   // rows per work-group and head of the group (scaled by g, capped)
+static inline int kv_tile_rows(int g) { return KV_TILE_ROWS * (g < 2 ? g : 2); }
 
 template <int D, int BK> struct KvCfg {
   static constexpr int NW = BK / 16;        // one wave per 16 keys
   static constexpr int NT = NW * 64;
-  static constexpr int QS = D + 8;          // LDS row stride of the Q / dO tiles
+  static constexpr int QS = D + 8;         // LDS row stride of the Q / dO tiles (16 B pad; a larger pad would push two work-groups past 160 KB of LDS)
   static constexpr int CPR = D / 8;         // 16-byte chunks per row
   static constexpr int CPT = KV_R * CPR / NT;  // chunks per thread and tensor
   static constexpr int ROW_STEP = NT / CPR;
@@ -90,7 +92,8 @@ template <int D, int BK> struct KvCfg {
   // with the fused dQ: K of the block (natural layout) and the dS^T tile [BK][KV_R]
   static constexpr int KS = D + 8;
   static constexpr int DSS = KV_R + 8;
-  static constexpr int BYTES_FUSED = BYTES + (BK * KS + BK * DSS) * 2;
+  static constexpr bool STAGE_DQ = BYTES + (BK * KS + BK * DSS + NW * 16 * QS) * 2 <= 160 * 1024;
+  static constexpr int BYTES_FUSED = BYTES + (BK * KS + BK * DSS + (STAGE_DQ ? NW * 16 * QS : 0)) * 2;  // + per-wave dQ staging tiles
   static constexpr int MIN_WAVES = (D <= 128 && NT <= 256) ? 2 : 1;  // work-groups per CU the registers allow
   static_assert(KV_R * CPR % NT == 0, "tile must divide evenly over the threads");
 };
@@ -113,6 +116,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   int* lim_s = reinterpret_cast<int*>(del_s + KV_R);
   T* Kl = reinterpret_cast<T*>(lim_s + KV_R);   // FUSE_DQ only
   T* dSs = Kl + BK * C::KS;                     // FUSE_DQ only
+  T* dQst = dSs + BK * C::DSS + (threadIdx.x >> 6) * (16 * C::QS);  // FUSE_DQ only: this wave's [16][D] tile
 
   const int h = blockIdx.y;
   const int64_t nbp1 = p.max_blocks + 1;
@@ -125,8 +129,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   const int rows = p.counts[h * p.max_blocks + gb] * p.g;
   const int start = MODE == KV_MODE_SELECTED ? p.starts[h * nbp1 + gb] : 0;
   const int ntile_b = tp[gb + 1] - tp[gb];
-  const int row_lo = (w - tp[gb]) * KV_TILE_ROWS;
-  const int row_hi = min(rows, row_lo + KV_TILE_ROWS);
+  const int row_lo = (w - tp[gb]) * p.kv_tile_rows;
+  const int row_hi = min(rows, row_lo + p.kv_tile_rows);
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int l16 = lane & 15, kg = lane >> 4;
@@ -304,8 +308,6 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 #pragma unroll
         for (int u = 0; u < BK / 32; ++u)
           dsb[u] = lds_read_tr8<T>(&dSs[32 * u * C::DSS + str_off + 16 * rt], 16 * C::DSS);
-        const int r = base + rt * 16 + l16;
-        T* orow = dqpart + (prow0 + r) * D + 4 * kg;
 #pragma unroll
         for (int t = 0; t < NDT; ++t) {
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -314,13 +316,27 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
             vec8 ka = lds_read_tr8<T>(&Kl[32 * u * C::KS + ktr_off + 16 * t], 16 * C::KS);
             acc = Elem<T>::mfma16(ka, dsb[u], acc);
           }
-          if (r < row_hi) {
-            vec4 x;
+          vec4 x;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) x[i] = (T)acc[i];
-            store8(orow + 16 * t, x);
+          for (int i = 0; i < 4; ++i) x[i] = (T)acc[i];
+          if (C::STAGE_DQ) {
+            store8(&dQst[l16 * QS + 16 * t + 4 * kg], x);
+          } else {  // LDS too small for the staging tiles: direct 8-byte stores
+            const int r = base + rt * 16 + l16;
+            if (r < row_hi) store8(dqpart + (prow0 + r) * D + 16 * t + 4 * kg, x);
           }
         }
+        // [16 rows][D] tile -> row-coalesced 16-byte stores (CPR lanes per row)
+        __builtin_amdgcn_wave_barrier();
+        constexpr int RPI = 64 / C::CPR;
+#pragma unroll
+        for (int j = 0; C::STAGE_DQ && j < 16 / RPI; ++j) {
+          const int row = lane / C::CPR + RPI * j;
+          const int r = base + rt * 16 + row;
+          vec8 x = load16<vec8>(&dQst[row * QS + (lane % C::CPR) * 8]);
+          if (r < row_hi) store16(dqpart + (prow0 + r) * D + (lane % C::CPR) * 8, x);
+        }
+        __builtin_amdgcn_wave_barrier();
       }
     }
     __syncthreads();

@@ -44,7 +44,9 @@ constexpr int SEL_TILE_ROWS = 8 * SEL_WG_ROWS;   // rows per work-group
 template <int D, int BK> struct SelLds {
   static constexpr int KS = D + 8;   // K row stride in elements (16 B pad: bank spread)
   static constexpr int VS = D + 16;  // V row stride in elements (32 B pad for the transposing reads)
-  static constexpr int BYTES = (BK * KS + BK * VS) * 2;
+  static constexpr int OS = D + 8;   // row stride of the per-wave output staging tile
+  static constexpr bool STAGE_OUT = (BK * KS + BK * VS + 4 * 32 * OS) * 2 <= 160 * 1024;
+  static constexpr int BYTES = (BK * KS + BK * VS + (STAGE_OUT ? 4 * 32 * OS : 0)) * 2;
   static constexpr int MIN_WAVES = (D <= 128 && BK <= 64) ? 2 : 1;  // waves per SIMD the register budget allows
 };
 
@@ -60,6 +62,8 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* Ks = reinterpret_cast<T*>(smem);
   T* Vs = Ks + BK * KS;
+  constexpr int OS = SelLds<D, BK>::OS;
+  T* Ost = Vs + BK * VS + (threadIdx.x >> 6) * (32 * OS);  // this wave's [32][D] staging tile
 
   const int h = blockIdx.y;
   const int64_t nbp1 = p.max_blocks + 1;
@@ -98,49 +102,54 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   const int lane = tid & 63, wv = tid >> 6;
   const int col = lane & 31, hh = lane >> 5;
   const int32_t* toks = p.sel_tokens + (int64_t)h * p.cap + start;
-  const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)h * p.g * p.q_sh + hh * (D / 2);
+  const T* qbase_row = reinterpret_cast<const T*>(p.q) + (int64_t)h * p.g * p.q_sh;
   const int64_t prow0 = ((int64_t)h * p.cap + start) * p.g;
   T* opart = reinterpret_cast<T*>(p.o_part);
   // this lane's address inside V for the transposing reads of O^T = V^T P^T:
   // keys 4*hh + (lane%16)/4 (+ 16*j, + 8), dims 16*((lane/16)&1) + 4*(lane%4) (+ 32*dt)
   const T* vtr = Vs + (4 * hh + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
-  // Software pipeline over the wave's 32-row sub-tiles: token ids are fetched
-  // two steps ahead, Q rows one step ahead of the MFMA work.
-  auto row_token = [&](int sub_, int& head_) {
+  // Pipeline over the wave's 32-row sub-tiles.  Q rows are fetched with row-coalesced
+  // 16-byte loads (CPR lanes cover one row, so a load instruction touches 8 cache lines
+  // instead of 64) one sub-tile ahead, parked in registers, and pass through the wave's
+  // LDS tile to reach the MFMA operand layout; token ids are fetched two steps ahead.
+  constexpr int CPR = D / 8;      // 16-byte chunks per row
+  constexpr int RPI = 64 / CPR;   // rows per load / store instruction
+  constexpr int NLD = 32 / RPI;   // instructions per 32-row tile
+  const int srow = lane / CPR, schunk = lane % CPR;
+  auto row_token = [&](int sub_) {  // token id of row (sub_ + col), kept by lane col
     const int r_ = min(sub_ + col, row_hi - 1);
-    const int trank_ = r_ / p.g;
-    head_ = r_ - trank_ * p.g;
-    return toks[trank_];
+    return toks[r_ / p.g];
   };
-  int sub = row_lo + wv * 32;
-  if (sub >= row_hi) return;
-  int head_n, head_nn = 0;
-  int tok_n = row_token(sub, head_n);
-  vec8 qnext[NKS];
-  {
-    const T* qrow = qbase + (int64_t)tok_n * p.q_sn + (int64_t)head_n * p.q_sh;
+  auto fetch_q = [&](vec8 (&dst)[NLD], int tok_lane, int sub_) {
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qnext[ks] = load16<vec8>(qrow + ks * 8);
-  }
-  int tok_nn = (sub + SEL_WG_ROWS < row_hi) ? row_token(sub + SEL_WG_ROWS, head_nn) : 0;
-
-  for (; sub < row_hi; sub += SEL_WG_ROWS) {
+    for (int j = 0; j < NLD; ++j) {
+      const int row = srow + RPI * j;
+      const int tok_ = __shfl(tok_lane, row, 64);
+      const int r_ = min(sub_ + row, row_hi - 1);
+      const int head_ = r_ % p.g;
+      dst[j] = load16<vec8>(qbase_row + (int64_t)tok_ * p.q_sn + (int64_t)head_ * p.q_sh + schunk * 8);
+    }
+  };
+  constexpr bool STAGED = SelLds<D, BK>::STAGE_OUT;  // false: LDS cannot hold the wave tiles, direct loads / stores
+  vec8 qst[NLD];
+  // one sub-tile: rows sub.. of the block; qst holds its Q rows (row-coalesced layout) on entry
+  // and those of the next sub-tile (token ids tok_next) on exit
+  auto step = [&](int token, int sub, int tok_next) {
     const int r = sub + col;
     const bool valid = r < row_hi;
-    const int token = tok_n;
-    vec8 qreg[NKS];
+    vec8 qdir[STAGED ? 1 : NKS];
+    if (STAGED) {
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qreg[ks] = qnext[ks];
-    tok_n = tok_nn;
-    head_n = head_nn;
-    if (sub + SEL_WG_ROWS < row_hi) {
-      const T* qrow = qbase + (int64_t)tok_n * p.q_sn + (int64_t)head_n * p.q_sh;
+      for (int j = 0; j < NLD; ++j) store16(&Ost[(srow + RPI * j) * OS + schunk * 8], qst[j]);
+      __builtin_amdgcn_wave_barrier();
+      if (sub + SEL_WG_ROWS < row_hi) fetch_q(qst, tok_next, sub + SEL_WG_ROWS);
+    } else {
+      const int head_ = min(r, row_hi - 1) % p.g;
+      const T* qrow = qbase_row + (int64_t)token * p.q_sn + (int64_t)head_ * p.q_sh + hh * (D / 2);
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) qnext[ks] = load16<vec8>(qrow + ks * 8);
+      for (int ks = 0; ks < NKS; ++ks) qdir[ks] = load16<vec8>(qrow + ks * 8);
     }
-    if (sub + 2 * SEL_WG_ROWS < row_hi) tok_nn = row_token(sub + 2 * SEL_WG_ROWS, head_nn);
-
     f32x16 acc[NA];
 #pragma unroll
     for (int a = 0; a < NA; ++a) {
@@ -149,9 +158,11 @@ selattn_fwd_main_kernel(SelFwdParams p) {
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         vec8 kf = load16<vec8>(&Ks[(a * 32 + col) * KS + hh * (D / 2) + ks * 8]);
-        acc[a] = Elem<T>::mfma32(kf, qreg[ks], acc[a]);
+        vec8 qf = STAGED ? load16<vec8>(&Ost[col * OS + hh * (D / 2) + ks * 8]) : qdir[STAGED ? 0 : ks];
+        acc[a] = Elem<T>::mfma32(kf, qf, acc[a]);
       }
     }
+    __builtin_amdgcn_wave_barrier();  // Q fragments consumed: the tile is reused for the output rows
     // causal mask: key index inside the block must be <= limit
     const int limit = (token - seq_start) - b_local * BK;
     float mx = -INFINITY;
@@ -179,11 +190,8 @@ selattn_fwd_main_kernel(SelFwdParams p) {
     l += xor32(l);
     const float inv_l = l > 0.f ? 1.f / l : 0.f;
     const int64_t prow = prow0 + r;
-    // Partial rows are stored in the lane-native order
-    //   pos = hh*(D/2) + dt*16 + i   <->   d = dt*32 + 8*(i/4) + 4*hh + i%4
-    // so that every lane owns one contiguous half row (16-byte stores); the
-    // merge kernel undoes the permutation when it writes O.
-    T* orow = opart + prow * D + hh * (D / 2);
+    // O^T accumulators -> this wave's LDS tile [row][d] -> 16-byte stores in which 16 lanes
+    // cover one full 2*D-byte row (8 cache lines per store instruction instead of 64)
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
       f32x16 oacc;
@@ -194,17 +202,41 @@ selattn_fwd_main_kernel(SelFwdParams p) {
         vec8 vf = lds_read_tr8<T>(vtr + 16 * j * VS + dt * 32, 8 * VS);
         oacc = Elem<T>::mfma32(vf, pk[j], oacc);
       }
-      if (valid) {
 #pragma unroll
-        for (int c8 = 0; c8 < 2; ++c8) {
-          vec8 x;
+      for (int qd = 0; qd < 4; ++qd) {
+        typename Elem<T>::vec4 x;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) x[e] = (T)(oacc[c8 * 8 + e] * inv_l);
-          store16(orow + dt * 16 + c8 * 8, x);
-        }
+        for (int e = 0; e < 4; ++e) x[e] = (T)(oacc[4 * qd + e] * inv_l);
+        if (SelLds<D, BK>::STAGE_OUT) store8(&Ost[col * OS + dt * 32 + 8 * qd + 4 * hh], x);
+        else if (valid) store8(opart + prow * D + dt * 32 + 8 * qd + 4 * hh, x);  // LDS too small: direct
       }
     }
+    __builtin_amdgcn_wave_barrier();
+    if (SelLds<D, BK>::STAGE_OUT) {
+      constexpr int CPR = D / 8;          // 16-byte chunks per row
+      constexpr int RPI = 64 / CPR;       // rows per store instruction
+      const int srow = lane / CPR, schunk = lane % CPR;
+#pragma unroll
+      for (int j = 0; j < 32 / RPI; ++j) {
+        const int row = srow + RPI * j;
+        vec8 x = load16<vec8>(&Ost[row * OS + schunk * 8]);
+        if (sub + row < row_hi) store16(opart + (prow0 + sub + row) * D + schunk * 8, x);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
     if (valid && hh == 0) p.lse_part[prow] = l > 0.f ? mref + log2f(l) : -INFINITY;
+  };
+
+  int sub = row_lo + wv * 32;
+  if (sub >= row_hi) return;
+  int ta = row_token(sub);
+  if (STAGED) fetch_q(qst, ta, sub);
+  int tb = sub + SEL_WG_ROWS < row_hi ? row_token(sub + SEL_WG_ROWS) : 0;
+  for (; sub < row_hi; sub += SEL_WG_ROWS) {
+    const int tc = sub + 2 * SEL_WG_ROWS < row_hi ? row_token(sub + 2 * SEL_WG_ROWS) : 0;
+    step(ta, sub, tb);
+    ta = tb;
+    tb = tc;
   }
 }
 
@@ -262,22 +294,10 @@ selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict_
       for (int e = 0; e < 8; ++e) accv[e] += wgt * (float)x[e];
     }
   }
-  // un-permute: positions [8*sub, 8*sub+8) of a partial row are two runs of 4 dims
-  {
-    typedef typename Elem<T>::vec4 vec4;
-    const int pos = sub * 8;
-    const int hh = pos / (D / 2), rem = pos % (D / 2);
-    const int dt = rem / 16, i0 = rem % 16;  // i0 in {0, 8}
-    T* orow = o + tok * o_sn + (int64_t)hq_i * o_sh + dt * 32 + 4 * hh + 8 * (i0 >> 2);
-    vec4 a, b;
+  vec8 out;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      a[e] = (T)accv[e];
-      b[e] = (T)accv[4 + e];
-    }
-    store8(orow, a);
-    store8(orow + 8, b);
-  }
+  for (int e = 0; e < 8; ++e) out[e] = (T)accv[e];
+  store16(o + tok * o_sn + (int64_t)hq_i * o_sh + sub * 8, out);
   if (sub == 0) lse[(int64_t)hq_i * n_tokens + tok] = lse_tot;
 }
 

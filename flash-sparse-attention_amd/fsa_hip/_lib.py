@@ -9,7 +9,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libfsa_gfx950.so")
+LIB_PATH = os.environ.get("FSA_HIP_LIBRARY") or os.path.join(_HERE, "libfsa_gfx950.so")
 
 _lib = None
 
