@@ -36,12 +36,15 @@ struct CmpParams {
   int64_t n_tokens;
   int g;
   int kernel_size, kernel_stride;
+  int window;  // sliding-window mode: key p visible to query i iff i - window <= p <= i
   float scale, scale_log2;
   // score / top-k
   float* score;        // [Hkv, N, score_ld]
   int64_t score_ld;
 };
 
+constexpr int CMP_MODE_COMPRESSED = 0;
+constexpr int CMP_MODE_WINDOW = 1;   // the same query-major kernels over raw keys with a causal band mask
 constexpr int CMP_BK = 64;      // compressed keys per tile
 constexpr int CMP_ROWS = 128;   // rows per work-group (4 waves x 32)
 
@@ -68,8 +71,20 @@ __device__ __forceinline__ void stage_kv_tile(const T* kbase, int64_t k_sn, cons
   }
 }
 
+// Per-row and per-work-group visible key range [lo, hi] (inclusive) in both modes.
+template <int MODE> struct KeyRange {
+  static __device__ __forceinline__ int hi(const CmpParams& p, int qi, int nc) {
+    if (MODE == CMP_MODE_WINDOW) return min(qi, nc - 1);
+    const int j = qi >= p.kernel_size - 1 ? (qi - p.kernel_size + 1) / p.kernel_stride : -1;
+    return min(j, nc - 1);
+  }
+  static __device__ __forceinline__ int lo(const CmpParams& p, int qi) {
+    return MODE == CMP_MODE_WINDOW ? max(0, qi - p.window) : 0;
+  }
+};
+
 // ---------------------------------------------------------------- forward ----
-template <typename T, int D>
+template <typename T, int D, int MODE>
 __global__ void __launch_bounds__(256)
 cmpattn_fwd_kernel(CmpParams p) {
   typedef typename Elem<T>::vec8 vec8;
@@ -82,7 +97,8 @@ cmpattn_fwd_kernel(CmpParams p) {
 
   const int s = blockIdx.y, h = blockIdx.z;
   const int q0 = p.cu_q[s], lq = p.cu_q[s + 1] - q0;
-  const int k0 = p.cu_k[s], nc = p.cu_k[s + 1] - k0;
+  const int k0 = MODE == CMP_MODE_WINDOW ? q0 : p.cu_k[s];
+  const int nc = MODE == CMP_MODE_WINDOW ? lq : p.cu_k[s + 1] - k0;
   const int rows_total = lq * p.g;
   const int row_lo = blockIdx.x * CMP_ROWS;
   if (row_lo >= rows_total) return;
@@ -97,11 +113,11 @@ cmpattn_fwd_kernel(CmpParams p) {
   vec8 qreg[NKS];
 #pragma unroll
   for (int ks = 0; ks < NKS; ++ks) qreg[ks] = load16<vec8>(qrow + ks * 8);
-  // last compressed key visible to this row, and to the last row of the work-group
-  int jmax = qi >= p.kernel_size - 1 ? (qi - p.kernel_size + 1) / p.kernel_stride : -1;
-  jmax = min(jmax, nc - 1);
-  const int qi_last = (min(rows_total, row_lo + CMP_ROWS) - 1) / p.g;
-  const int n_keys = qi_last >= p.kernel_size - 1 ? min(nc, (qi_last - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
+  // keys visible to this row and to the rows of the work-group
+  const int jmax = KeyRange<MODE>::hi(p, qi, nc), jmin = KeyRange<MODE>::lo(p, qi);
+  const int qi_first = row_lo / p.g, qi_last = (min(rows_total, row_lo + CMP_ROWS) - 1) / p.g;
+  const int n_keys = KeyRange<MODE>::hi(p, qi_last, nc) + 1;                 // end of the work-group's key range
+  const int jt0 = KeyRange<MODE>::lo(p, qi_first) / CMP_BK * CMP_BK;          // its tile-aligned start
 
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
@@ -114,8 +130,8 @@ cmpattn_fwd_kernel(CmpParams p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
 
-  for (int jt = 0; jt < n_keys; jt += CMP_BK) {
-    if (jt) __syncthreads();
+  for (int jt = jt0; jt < n_keys; jt += CMP_BK) {
+    if (jt != jt0) __syncthreads();
     stage_kv_tile<T, D>(kbase, p.k_sn, vbase, p.v_sn, k0 + jt, nc - jt, Ks, Vs, tid);
     __syncthreads();
     f32x16 acc[NA];
@@ -129,14 +145,14 @@ cmpattn_fwd_kernel(CmpParams p) {
         acc[a] = Elem<T>::mfma32(kf, qreg[ks], acc[a]);
       }
     }
-    const int limit = jmax - jt;
+    const int limit = jmax - jt, limit_lo = jmin - jt;
     float mx = m;
 #pragma unroll
     for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-        const float sv = key <= limit ? acc[a][i] : -INFINITY;
+        const float sv = (key <= limit && key >= limit_lo) ? acc[a][i] : -INFINITY;
         acc[a][i] = sv;
         mx = fmaxf(mx, sv);
       }
@@ -183,7 +199,7 @@ cmpattn_fwd_kernel(CmpParams p) {
 }
 
 // --------------------------------------------------------------------- dq ----
-template <typename T, int D>
+template <typename T, int D, int MODE>
 __global__ void __launch_bounds__(256)
 cmpattn_bwd_dq_kernel(CmpParams p) {
   typedef typename Elem<T>::vec8 vec8;
@@ -196,7 +212,8 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
 
   const int s = blockIdx.y, h = blockIdx.z;
   const int q0 = p.cu_q[s], lq = p.cu_q[s + 1] - q0;
-  const int k0 = p.cu_k[s], nc = p.cu_k[s + 1] - k0;
+  const int k0 = MODE == CMP_MODE_WINDOW ? q0 : p.cu_k[s];
+  const int nc = MODE == CMP_MODE_WINDOW ? lq : p.cu_k[s + 1] - k0;
   const int rows_total = lq * p.g;
   const int row_lo = blockIdx.x * CMP_ROWS;
   if (row_lo >= rows_total) return;
@@ -218,10 +235,10 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
   const int64_t stat = (int64_t)hq_i * p.n_tokens + q0 + qi;
   const float lse_r = p.lse[stat];
   const float delta_r = p.delta[stat];
-  int jmax = qi >= p.kernel_size - 1 ? (qi - p.kernel_size + 1) / p.kernel_stride : -1;
-  jmax = min(jmax, nc - 1);
-  const int qi_last = (min(rows_total, row_lo + CMP_ROWS) - 1) / p.g;
-  const int n_keys = qi_last >= p.kernel_size - 1 ? min(nc, (qi_last - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
+  const int jmax = KeyRange<MODE>::hi(p, qi, nc), jmin = KeyRange<MODE>::lo(p, qi);
+  const int qi_first = row_lo / p.g, qi_last = (min(rows_total, row_lo + CMP_ROWS) - 1) / p.g;
+  const int n_keys = KeyRange<MODE>::hi(p, qi_last, nc) + 1;                 // end of the work-group's key range
+  const int jt0 = KeyRange<MODE>::lo(p, qi_first) / CMP_BK * CMP_BK;          // its tile-aligned start
 
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
@@ -233,8 +250,8 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) dacc[dt][i] = 0.f;
 
-  for (int jt = 0; jt < n_keys; jt += CMP_BK) {
-    if (jt) __syncthreads();
+  for (int jt = jt0; jt < n_keys; jt += CMP_BK) {
+    if (jt != jt0) __syncthreads();
     stage_kv_tile<T, D>(kbase, p.k_sn, vbase, p.v_sn, k0 + jt, nc - jt, Ks, Vs, tid);
     __syncthreads();
     f32x16 acc[NA], dp[NA];
@@ -253,14 +270,14 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
         dp[a] = Elem<T>::mfma32(vf, doreg[ks], dp[a]);
       }
     }
-    const int limit = jmax - jt;
+    const int limit = jmax - jt, limit_lo = jmin - jt;
     vec8 dsk[NJ];
 #pragma unroll
     for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-        const float pv = key <= limit ? exp2f(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
+        const float pv = (key <= limit && key >= limit_lo) ? exp2f(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
         dsk[a * 2 + (i >> 3)][i & 7] = (T)(pv * (dp[a][i] - delta_r) * p.scale);
       }
 #pragma unroll
@@ -327,6 +344,33 @@ __global__ void cmp_kv_blocks_kernel(const int32_t* __restrict__ cu_q, const int
       const int s = upper_seg(cu_tiles, batch, (int)gb);
       const int q_first = (int)(gb - cu_tiles[s]) * CMP_BK * kernel_stride + kernel_size - 1;
       c = max(0, cu_q[s + 1] - cu_q[s] - q_first);
+    }
+    for (int h = 0; h < hkv; ++h) counts[h * max_blocks + gb] = c;
+  }
+}
+
+// work list of the dK/dV kernel in sliding-window mode: one "block" per tile of 64 keys (tokens);
+// its rows are the queries from the tile's first key to window tokens past its last key
+__global__ void win_kv_blocks_kernel(const int32_t* __restrict__ cu_q, int batch, int hkv, int64_t max_blocks,
+                                     int window, int32_t* __restrict__ cu_tiles, int32_t* __restrict__ counts) {
+  __shared__ int total;
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    cu_tiles[0] = 0;
+    for (int s = 0; s < batch; ++s) {
+      acc += (cu_q[s + 1] - cu_q[s] + CMP_BK - 1) / CMP_BK;
+      cu_tiles[s + 1] = acc;
+    }
+    total = acc;
+  }
+  __syncthreads();
+  for (int64_t gb = threadIdx.x; gb < max_blocks; gb += blockDim.x) {
+    int c = 0;
+    if (gb < total) {
+      const int s = upper_seg(cu_tiles, batch, (int)gb);
+      const int len = cu_q[s + 1] - cu_q[s];
+      const int first = (int)(gb - cu_tiles[s]) * CMP_BK;
+      c = max(0, min(len, first + CMP_BK + window) - first);
     }
     for (int h = 0; h < hkv; ++h) counts[h * max_blocks + gb] = c;
   }
@@ -523,45 +567,65 @@ static CmpBwdWs cmp_bwd_ws(int64_t n, int64_t n_k, int64_t max_q, int batch, int
   return w;
 }
 
-template <typename T, int D>
-static int cmp_fwd_launch(const CmpParams& p, int batch, int hkv, int64_t max_rows, hipStream_t stream) {
-  int rc = cmp_set_lds(cmpattn_fwd_kernel<T, D>, CmpLds<D>::BYTES);
+template <typename T, int D, int MODE>
+static int attn_fwd_launch(const CmpParams& p, int batch, int hkv, int64_t max_rows, hipStream_t stream) {
+  int rc = cmp_set_lds(cmpattn_fwd_kernel<T, D, MODE>, CmpLds<D>::BYTES);
   if (rc) return rc;
   dim3 grid((unsigned)((max_rows + CMP_ROWS - 1) / CMP_ROWS), batch, hkv);
-  ProfScope ps_("cmpattn_fwd", stream);
-  cmpattn_fwd_kernel<T, D><<<grid, 256, CmpLds<D>::BYTES, stream>>>(p);
+  ProfScope ps_(MODE == CMP_MODE_WINDOW ? "winattn_fwd" : "cmpattn_fwd", stream);
+  cmpattn_fwd_kernel<T, D, MODE><<<grid, 256, CmpLds<D>::BYTES, stream>>>(p);
+  return 0;
+}
+template <typename T, int D>
+static int cmp_fwd_launch(const CmpParams& p, int batch, int hkv, int64_t max_rows, hipStream_t stream) {
+  return attn_fwd_launch<T, D, CMP_MODE_COMPRESSED>(p, batch, hkv, max_rows, stream);
+}
+template <typename T, int D>
+static int win_fwd_launch(const CmpParams& p, int batch, int hkv, int64_t max_rows, hipStream_t stream) {
+  return attn_fwd_launch<T, D, CMP_MODE_WINDOW>(p, batch, hkv, max_rows, stream);
+}
+
+template <typename T, int D, int MODE>
+static int attn_bwd_launch(const CmpParams& p, const SelBwdParams& kv, int batch, int hq, int hkv,
+                           int64_t max_rows, int64_t n, hipStream_t stream) {
+  constexpr int KVM = MODE == CMP_MODE_WINDOW ? KV_MODE_WINDOW : KV_MODE_COMPRESSED;
+  int rc = cmp_set_lds(cmpattn_bwd_dq_kernel<T, D, MODE>, CmpLds<D>::BYTES);
+  if (rc) return rc;
+  rc = cmp_set_lds(attn_bwd_dkdv_kernel<T, D, CMP_BK, KVM>, KvCfg<D, CMP_BK>::BYTES);
+  if (rc) return rc;
+  {
+    ProfScope ps_(MODE == CMP_MODE_WINDOW ? "winattn_bwd_delta" : "cmpattn_bwd_delta", stream);
+    constexpr int RPB = 256 / (D / 8);
+    cmp_delta_kernel<T, D><<<(unsigned)((n * hq + RPB - 1) / RPB), 256, 0, stream>>>(
+        (const T*)p.o, p.o_sn, p.o_sh, (const T*)p.d_o, p.do_sn, p.do_sh, n, hq, (float*)p.delta);
+  }
+  {
+    ProfScope ps_(MODE == CMP_MODE_WINDOW ? "winattn_bwd_dq" : "cmpattn_bwd_dq", stream);
+    dim3 grid((unsigned)((max_rows + CMP_ROWS - 1) / CMP_ROWS), batch, hkv);
+    cmpattn_bwd_dq_kernel<T, D, MODE><<<grid, 256, CmpLds<D>::BYTES, stream>>>(p);
+  }
+  {
+    ProfScope ps_(MODE == CMP_MODE_WINDOW ? "winattn_bwd_dkdv" : "cmpattn_bwd_dkdv", stream);
+    attn_bwd_dkdv_kernel<T, D, CMP_BK, KVM>
+        <<<dim3((unsigned)kv.max_tiles, hkv), KvCfg<D, CMP_BK>::NT, KvCfg<D, CMP_BK>::BYTES, stream>>>(kv);
+  }
+  {
+    ProfScope ps_(MODE == CMP_MODE_WINDOW ? "winattn_bwd_dkdv_reduce" : "cmpattn_bwd_dkdv_reduce", stream);
+    attn_bwd_dkdv_reduce_kernel<T, D, CMP_BK, KVM>
+        <<<dim3((unsigned)kv.max_blocks, hkv), 256, 0, stream>>>(kv);
+  }
   return 0;
 }
 
 template <typename T, int D>
 static int cmp_bwd_launch(const CmpParams& p, const SelBwdParams& kv, int batch, int hq, int hkv,
                           int64_t max_rows, int64_t n, hipStream_t stream) {
-  int rc = cmp_set_lds(cmpattn_bwd_dq_kernel<T, D>, CmpLds<D>::BYTES);
-  if (rc) return rc;
-  rc = cmp_set_lds(attn_bwd_dkdv_kernel<T, D, CMP_BK, KV_MODE_COMPRESSED>, KvCfg<D, CMP_BK>::BYTES);
-  if (rc) return rc;
-  {
-    ProfScope ps_("cmpattn_bwd_delta", stream);
-    constexpr int RPB = 256 / (D / 8);
-    cmp_delta_kernel<T, D><<<(unsigned)((n * hq + RPB - 1) / RPB), 256, 0, stream>>>(
-        (const T*)p.o, p.o_sn, p.o_sh, (const T*)p.d_o, p.do_sn, p.do_sh, n, hq, (float*)p.delta);
-  }
-  {
-    ProfScope ps_("cmpattn_bwd_dq", stream);
-    dim3 grid((unsigned)((max_rows + CMP_ROWS - 1) / CMP_ROWS), batch, hkv);
-    cmpattn_bwd_dq_kernel<T, D><<<grid, 256, CmpLds<D>::BYTES, stream>>>(p);
-  }
-  {
-    ProfScope ps_("cmpattn_bwd_dkdv", stream);
-    attn_bwd_dkdv_kernel<T, D, CMP_BK, KV_MODE_COMPRESSED>
-        <<<dim3((unsigned)kv.max_tiles, hkv), KvCfg<D, CMP_BK>::NT, KvCfg<D, CMP_BK>::BYTES, stream>>>(kv);
-  }
-  {
-    ProfScope ps_("cmpattn_bwd_dkdv_reduce", stream);
-    attn_bwd_dkdv_reduce_kernel<T, D, CMP_BK, KV_MODE_COMPRESSED>
-        <<<dim3((unsigned)kv.max_blocks, hkv), 256, 0, stream>>>(kv);
-  }
-  return 0;
+  return attn_bwd_launch<T, D, CMP_MODE_COMPRESSED>(p, kv, batch, hq, hkv, max_rows, n, stream);
+}
+template <typename T, int D>
+static int win_bwd_launch(const CmpParams& p, const SelBwdParams& kv, int batch, int hq, int hkv,
+                          int64_t max_rows, int64_t n, hipStream_t stream) {
+  return attn_bwd_launch<T, D, CMP_MODE_WINDOW>(p, kv, batch, hq, hkv, max_rows, n, stream);
 }
 
 template <typename T, int D>
@@ -594,6 +658,14 @@ static int cmp_fwd_dispatch(int dtype, int head_dim, const CmpParams& p, int bat
 static int cmp_bwd_dispatch(int dtype, int head_dim, const CmpParams& p, const SelBwdParams& kv, int batch,
                             int hq, int hkv, int64_t max_rows, int64_t n, hipStream_t stream) {
   FSA_CMP_DISPATCH(cmp_bwd_launch, p, kv, batch, hq, hkv, max_rows, n, stream);
+}
+static int win_fwd_dispatch(int dtype, int head_dim, const CmpParams& p, int batch, int hkv,
+                            int64_t max_rows, hipStream_t stream) {
+  FSA_CMP_DISPATCH(win_fwd_launch, p, batch, hkv, max_rows, stream);
+}
+static int win_bwd_dispatch(int dtype, int head_dim, const CmpParams& p, const SelBwdParams& kv, int batch,
+                            int hq, int hkv, int64_t max_rows, int64_t n, hipStream_t stream) {
+  FSA_CMP_DISPATCH(win_bwd_launch, p, kv, batch, hq, hkv, max_rows, n, stream);
 }
 static int cmp_score_dispatch(int dtype, int head_dim, const CmpParams& p, int batch, int hkv,
                               int64_t max_q, hipStream_t stream) {
@@ -763,5 +835,103 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
     cmp_topk_kernel<<<(unsigned)((rows + 3) / 4), 256, (size_t)4 * nblk * 4, stream>>>(tp);
   }
   FSA_CHECK_LAUNCH("fsa_cmp_topk select");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Sliding-window attention (causal band of `window` + 1 keys): the third branch of the module.
+extern "C" int fsa_winattn_fwd(const void* q, const void* k, const void* v, int32_t dtype,
+                               int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n,
+                               int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                               const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                               int64_t max_seqlen, int32_t num_q_heads, int32_t num_kv_heads,
+                               int32_t head_dim, int32_t window, float softmax_scale, void* o,
+                               int64_t o_stride_n, int64_t o_stride_h, float* lse, void* stream_) {
+  FSA_CHECK_ARG(q && k && v && o && lse && cu_seqlens, "fsa_winattn_fwd: null pointer");
+  int rc = cmp_check_common("fsa_winattn_fwd", dtype, num_q_heads, num_kv_heads, 1, 1, batch, total_tokens);
+  if (rc) return rc;
+  FSA_CHECK_ARG(window >= 0 && max_seqlen >= 1 && max_seqlen <= total_tokens, "fsa_winattn_fwd: bad sizes");
+  CmpParams p = {};
+  p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse;
+  p.q_sn = q_stride_n; p.q_sh = q_stride_h; p.k_sn = k_stride_n; p.k_sh = k_stride_h;
+  p.v_sn = v_stride_n; p.v_sh = v_stride_h; p.o_sn = o_stride_n; p.o_sh = o_stride_h;
+  p.cu_q = cu_seqlens; p.cu_k = cu_seqlens; p.n_tokens = total_tokens;
+  p.g = num_q_heads / num_kv_heads; p.kernel_size = 1; p.kernel_stride = 1; p.window = window;
+  p.scale = softmax_scale; p.scale_log2 = softmax_scale * LOG2E;
+  rc = win_fwd_dispatch(dtype, head_dim, p, batch, num_kv_heads, max_seqlen * p.g, (hipStream_t)stream_);
+  if (rc) return rc;
+  FSA_CHECK_LAUNCH("fsa_winattn_fwd");
+  return 0;
+}
+
+static CmpBwdWs win_bwd_ws(int64_t n, int64_t max_q, int window, int batch, int hq, int hkv, int d) {
+  CmpBwdWs w = cmp_bwd_ws(n, n, max_q, batch, hq, hkv, d);
+  const int g = hq / hkv;
+  const int64_t rows = (int64_t)(CMP_BK + window) * g;
+  w.max_tiles = w.max_blocks * ((rows + kv_tile_rows(g) - 1) / kv_tile_rows(g) + 1);
+  w.total = w.off_part + align_up((size_t)hkv * w.max_tiles * 2 * CMP_BK * d * 4, 256);
+  return w;
+}
+
+extern "C" size_t fsa_winattn_bwd_workspace_bytes(int64_t total_tokens, int64_t max_seqlen, int32_t window,
+                                                  int32_t batch, int32_t num_q_heads,
+                                                  int32_t num_kv_heads, int32_t head_dim) {
+  return win_bwd_ws(total_tokens, max_seqlen, window, batch, num_q_heads, num_kv_heads, head_dim).total;
+}
+
+extern "C" int fsa_winattn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                               const float* lse, int32_t dtype, int64_t q_stride_n, int64_t q_stride_h,
+                               int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n,
+                               int64_t v_stride_h, int64_t o_stride_n, int64_t o_stride_h,
+                               int64_t do_stride_n, int64_t do_stride_h, const int32_t* cu_seqlens,
+                               int32_t batch, int64_t total_tokens, int64_t max_seqlen,
+                               int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                               int32_t window, float softmax_scale, void* dq, void* dk, void* dv,
+                               void* workspace, size_t workspace_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FSA_CHECK_ARG(q && k && v && o && d_o && lse && dq && dk && dv && cu_seqlens, "fsa_winattn_bwd: null pointer");
+  int rc = cmp_check_common("fsa_winattn_bwd", dtype, num_q_heads, num_kv_heads, 1, 1, batch, total_tokens);
+  if (rc) return rc;
+  FSA_CHECK_ARG(window >= 0 && max_seqlen >= 1 && max_seqlen <= total_tokens, "fsa_winattn_bwd: bad sizes");
+  CmpBwdWs ws = win_bwd_ws(total_tokens, max_seqlen, window, batch, num_q_heads, num_kv_heads, head_dim);
+  if (!workspace || workspace_bytes < ws.total) {
+    set_error("fsa_winattn_bwd: workspace too small (%zu < %zu)", workspace_bytes, ws.total);
+    return FSA_ERR_WORKSPACE;
+  }
+  char* wsp = (char*)workspace;
+  const int g = num_q_heads / num_kv_heads;
+  float* delta = (float*)(wsp + ws.off_delta);
+  int32_t* cu_tiles = (int32_t*)(wsp + ws.off_cu_tiles);
+  int32_t* counts = (int32_t*)(wsp + ws.off_counts);
+  int32_t* tile_prefix = (int32_t*)(wsp + ws.off_tiles);
+  win_kv_blocks_kernel<<<1, 256, 0, stream>>>(cu_seqlens, batch, num_kv_heads, ws.max_blocks, window, cu_tiles,
+                                              counts);
+  rc = fsa_build_tiles(counts, num_kv_heads, ws.max_blocks, g, kv_tile_rows(g), tile_prefix, stream_);
+  if (rc) return rc;
+
+  CmpParams p = {};
+  p.q = q; p.k = k; p.v = v; p.o = (void*)o; p.d_o = d_o; p.dq = dq; p.lse = (float*)lse; p.delta = delta;
+  p.q_sn = q_stride_n; p.q_sh = q_stride_h; p.k_sn = k_stride_n; p.k_sh = k_stride_h;
+  p.v_sn = v_stride_n; p.v_sh = v_stride_h; p.o_sn = o_stride_n; p.o_sh = o_stride_h;
+  p.do_sn = do_stride_n; p.do_sh = do_stride_h;
+  p.cu_q = cu_seqlens; p.cu_k = cu_seqlens; p.n_tokens = total_tokens;
+  p.g = g; p.kernel_size = 1; p.kernel_stride = 1; p.window = window;
+  p.scale = softmax_scale; p.scale_log2 = softmax_scale * LOG2E;
+
+  SelBwdParams kv = {};
+  kv.q = q; kv.k = k; kv.v = v; kv.d_o = d_o; kv.lse = lse; kv.delta = delta;
+  kv.q_sn = q_stride_n; kv.q_sh = q_stride_h; kv.k_sn = k_stride_n; kv.k_sh = k_stride_h;
+  kv.v_sn = v_stride_n; kv.v_sh = v_stride_h; kv.do_sn = do_stride_n; kv.do_sh = do_stride_h;
+  kv.cu_seqlens = cu_seqlens; kv.cu_blocks = cu_tiles; kv.counts = counts; kv.tile_prefix = tile_prefix;
+  kv.batch = batch; kv.max_blocks = ws.max_blocks; kv.n_tokens = total_tokens; kv.g = g;
+  kv.scale = softmax_scale; kv.scale_log2 = softmax_scale * LOG2E;
+  kv.dkdv_part = (float*)(wsp + ws.off_part); kv.max_tiles = ws.max_tiles; kv.kv_tile_rows = kv_tile_rows(g);
+  kv.dk = dk; kv.dv = dv; kv.dk_sn = (int64_t)num_kv_heads * head_dim; kv.dk_sh = head_dim;
+  kv.cu_seqlens_k = cu_seqlens; kv.kernel_size = 1; kv.kernel_stride = 1; kv.window = window;
+
+  rc = win_bwd_dispatch(dtype, head_dim, p, kv, batch, num_q_heads, num_kv_heads, max_seqlen * g, total_tokens,
+                        stream);
+  if (rc) return rc;
+  FSA_CHECK_LAUNCH("fsa_winattn_bwd");
   return 0;
 }

@@ -43,11 +43,13 @@ struct SelBwdParams {
   // compressed-attention mode only
   const int32_t* cu_seqlens_k;
   int kernel_size, kernel_stride;
+  int window;  // sliding-window mode only
 };
 
 
 constexpr int KV_MODE_SELECTED = 0;
 constexpr int KV_MODE_COMPRESSED = 1;
+constexpr int KV_MODE_WINDOW = 2;  // sliding window: key p visible to query i iff i - window <= p <= i
 
 // What a "block" of the work list is in each mode.
 template <int MODE, int BK> struct KvBlock {
@@ -61,6 +63,11 @@ template <int MODE, int BK> struct KvBlock {
       n_keys_valid = p.cu_seqlens[s + 1] - key_row0;       // may exceed BK
       q_first = 0;
       key_base = b_local * BK;                             // position of key 0 of the block
+    } else if (MODE == KV_MODE_WINDOW) {
+      key_row0 = seq_start + b_local * BK;
+      n_keys_valid = p.cu_seqlens[s + 1] - key_row0;
+      q_first = b_local * BK;                              // a key is first seen by the query at its own position
+      key_base = b_local * BK;
     } else {
       const int k0 = p.cu_seqlens_k[s];
       key_row0 = k0 + b_local * BK;                        // K/V rows are compressed tokens
@@ -71,8 +78,13 @@ template <int MODE, int BK> struct KvBlock {
   }
   // number of keys of the block visible to the query at sequence-local position qpos, minus one
   __device__ __forceinline__ int limit(const SelBwdParams& p, int qpos) const {
-    if (MODE == KV_MODE_SELECTED) return qpos - key_base;
+    if (MODE == KV_MODE_SELECTED || MODE == KV_MODE_WINDOW) return qpos - key_base;
     return (qpos - p.kernel_size + 1) / p.kernel_stride - key_base;  // qpos >= q_first >= ks-1
+  }
+  // first key of the block (index inside the block) visible to that query
+  __device__ __forceinline__ int limit_lo(const SelBwdParams& p, int qpos) const {
+    if (MODE == KV_MODE_WINDOW) return qpos - p.window - key_base;
+    return -(1 << 30);
   }
 };
 
@@ -88,7 +100,7 @@ template <int D, int BK> struct KvCfg {
   static constexpr int CPR = D / 8;         // 16-byte chunks per row
   static constexpr int CPT = KV_R * CPR / NT;  // chunks per thread and tensor
   static constexpr int ROW_STEP = NT / CPR;
-  static constexpr int BYTES = 2 * KV_R * QS * 2 + KV_R * 12;
+  static constexpr int BYTES = 2 * KV_R * QS * 2 + KV_R * 16;
   // with the fused dQ: K of the block (natural layout) and the dS^T tile [BK][KV_R]
   static constexpr int KS = D + 8;
   static constexpr int DSS = KV_R + 8;
@@ -114,7 +126,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   float* lse_s = reinterpret_cast<float*>(Os + KV_R * QS);
   float* del_s = lse_s + KV_R;
   int* lim_s = reinterpret_cast<int*>(del_s + KV_R);
-  T* Kl = reinterpret_cast<T*>(lim_s + KV_R);   // FUSE_DQ only
+  int* llo_s = lim_s + KV_R;
+  T* Kl = reinterpret_cast<T*>(llo_s + KV_R);   // FUSE_DQ only
   T* dSs = Kl + BK * C::KS;                     // FUSE_DQ only
   T* dQst = dSs + BK * C::DSS + (threadIdx.x >> 6) * (16 * C::QS);  // FUSE_DQ only: this wave's [16][D] tile
 
@@ -175,7 +188,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 
   vec8 qst[C::CPT], dost[C::CPT];
   float lse_st = 0.f, del_st = 0.f;
-  int lim_st = 0;
+  int lim_st = 0, llo_st = 0;
   int tok_pf[C::CPT], tok_stat = 0;  // token ids of the pass after the one being fetched
   auto fetch_tokens = [&](int base) {
 #pragma unroll
@@ -204,6 +217,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       lse_st = INFINITY;  // rows past the end: P = exp2(s - inf) = 0
       del_st = 0.f;
       lim_st = -1;
+      llo_st = 0;
       if (r < row_hi) {
         const int trank = r / p.g, head = r - trank * p.g;
         const int token = tok_stat;
@@ -211,6 +225,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         lse_st = p.lse[stat];
         del_st = p.delta[stat];
         lim_st = blk.limit(p, token - blk.seq_start);
+        llo_st = blk.limit_lo(p, token - blk.seq_start);
       }
     }
   };
@@ -225,6 +240,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       lse_s[tid] = lse_st;
       del_s[tid] = del_st;
       lim_s[tid] = lim_st;
+      llo_s[tid] = llo_st;
     }
   };
 
@@ -270,9 +286,15 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       const float lse_r[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
       const float del_r[4] = {del4.x, del4.y, del4.z, del4.w};
       const int lim_r[4] = {lim4.x, lim4.y, lim4.z, lim4.w};
+      int llo_r[4] = {0, 0, 0, 0};
+      if (MODE == KV_MODE_WINDOW) {
+        const int4 llo4 = *reinterpret_cast<const int4*>(&llo_s[rt * 16 + 4 * kg]);
+        llo_r[0] = llo4.x; llo_r[1] = llo4.y; llo_r[2] = llo4.z; llo_r[3] = llo4.w;
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = key <= lim_r[i] ? exp2f(sacc[i] * p.scale_log2 - lse_r[i]) : 0.f;
+        const bool vis = key <= lim_r[i] && (MODE != KV_MODE_WINDOW || key >= llo_r[i]);
+        const float pv = vis ? exp2f(sacc[i] * p.scale_log2 - lse_r[i]) : 0.f;
         const float ds = pv * (dpacc[i] - del_r[i]) * p.scale;
         pk[rt][i] = (T)pv;
         dsk[rt][i] = (T)ds;

@@ -50,6 +50,13 @@ SIGNATURES = {
     "fsa_cmp_topk": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, vp, vp, i32,
                                i64, i64, i64, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, f32,
                                vp, vp, vp, sz, vp]),
+    "fsa_winattn_fwd": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, i32, i64, i64,
+                                  i32, i32, i32, i32, f32, vp, i64, i64, vp, vp]),
+    "fsa_winattn_bwd_workspace_bytes": (sz, [i64, i64, i32, i32, i32, i32, i32]),
+    "fsa_winattn_bwd": (C.c_int, [vp, vp, vp, vp, vp, vp, i32,
+                                  i64, i64, i64, i64, i64, i64, i64, i64, i64, i64,
+                                  vp, i32, i64, i64, i32, i32, i32, i32, f32,
+                                  vp, vp, vp, vp, sz, vp]),
     "fsa_decode_cmpattn": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp,
                                      i32, i32, i32, i32, i32, i32, f32, i32, vp, vp, vp, i64, vp]),
     "fsa_decode_topk": (C.c_int, [vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,

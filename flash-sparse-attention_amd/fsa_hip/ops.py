@@ -299,3 +299,47 @@ def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scal
                                 float(softmax_scale), _ptr(o), _ptr(lse), _stream(dev))
     _lib.check(rc, "fsa_decode_selattn")
     return o, lse
+
+
+def winattn_fwd(q, k, v, cu_seqlens, max_seqlen, window, softmax_scale=None):
+    """Causal sliding-window attention (keys i-window..i): (o, lse [Hq,N] fp32 base 2)."""
+    _check_qkv(q, k, v)
+    lib = _lib.load()
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    o = torch.empty((n, hq, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((hq, n), dtype=torch.float32, device=q.device)
+    rc = lib.fsa_winattn_fwd(_ptr(q), _ptr(k), _ptr(v), _DTYPE[q.dtype], q.stride(0), q.stride(1), k.stride(0),
+                             k.stride(1), v.stride(0), v.stride(1), _ptr(cu_seqlens), cu_seqlens.numel() - 1, n,
+                             int(max_seqlen), hq, hkv, d, int(window), float(softmax_scale), _ptr(o), o.stride(0),
+                             o.stride(1), _ptr(lse), _stream(q.device))
+    _lib.check(rc, "fsa_winattn_fwd")
+    return o, lse
+
+
+def winattn_bwd(q, k, v, o, do, lse, cu_seqlens, max_seqlen, window, softmax_scale=None):
+    """Backward of winattn_fwd: (dq, dk, dv)."""
+    _check_qkv(q, k, v)
+    lib = _lib.load()
+    n, hq, d = q.shape
+    hkv = k.shape[1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    if do.stride(2) != 1:
+        do = do.contiguous()
+    dev = q.device
+    dq = torch.empty((n, hq, d), dtype=q.dtype, device=dev)
+    dk = torch.empty((n, hkv, d), dtype=q.dtype, device=dev)
+    dv = torch.empty((n, hkv, d), dtype=q.dtype, device=dev)
+    batch = cu_seqlens.numel() - 1
+    ws_bytes = lib.fsa_winattn_bwd_workspace_bytes(n, int(max_seqlen), int(window), batch, hq, hkv, d)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    rc = lib.fsa_winattn_bwd(_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _DTYPE[q.dtype],
+                             q.stride(0), q.stride(1), k.stride(0), k.stride(1), v.stride(0), v.stride(1),
+                             o.stride(0), o.stride(1), do.stride(0), do.stride(1), _ptr(cu_seqlens), batch, n,
+                             int(max_seqlen), hq, hkv, d, int(window), float(softmax_scale), _ptr(dq), _ptr(dk),
+                             _ptr(dv), _ptr(ws), ws_bytes, _stream(dev))
+    _lib.check(rc, "fsa_winattn_bwd")
+    return dq, dk, dv

@@ -248,6 +248,34 @@ int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, 
                        int32_t head_dim, int32_t topk, int32_t block_size, float softmax_scale, void* o,
                        float* lse, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Sliding-window attention: the query at sequence-local position i attends the
+ * keys p with i - window <= p <= i of its own sequence (window + 1 keys).
+ * Replaces flash_attn_varlen_func(causal=True, window_size=(window, -1)) in
+ * fsa/module/fsa.py:149-159 (a third-party kernel in the reference).  Same
+ * layouts as selected attention; dq contiguous [N,Hq,D], dk/dv contiguous
+ * [N,Hkv,D]; max_seqlen is an upper bound of the longest sequence.
+ * ---------------------------------------------------------------------- */
+int fsa_winattn_fwd(const void* q, const void* k, const void* v, int32_t dtype,
+                    int64_t q_stride_n, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                    int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_seqlens, int32_t batch,
+                    int64_t total_tokens, int64_t max_seqlen, int32_t num_q_heads, int32_t num_kv_heads,
+                    int32_t head_dim, int32_t window, float softmax_scale, void* o, int64_t o_stride_n,
+                    int64_t o_stride_h, float* lse, void* stream);
+
+size_t fsa_winattn_bwd_workspace_bytes(int64_t total_tokens, int64_t max_seqlen, int32_t window,
+                                       int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                       int32_t head_dim);
+
+int fsa_winattn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                    const float* lse, int32_t dtype, int64_t q_stride_n, int64_t q_stride_h,
+                    int64_t k_stride_n, int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                    int64_t o_stride_n, int64_t o_stride_h, int64_t do_stride_n, int64_t do_stride_h,
+                    const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens, int64_t max_seqlen,
+                    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t window,
+                    float softmax_scale, void* dq, void* dk, void* dv, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,92 @@
+"""Pins the module-side oracle pieces (window attention, rope tables, rotary)."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import module as orc
+
+
+def test_window_attention_matches_sdpa_band_mask():
+    gen = torch.Generator().manual_seed(0)
+    cu = [0, 70, 71, 200]
+    q = torch.randn(200, 4, 16, generator=gen, dtype=torch.float64)
+    k = torch.randn(200, 2, 16, generator=gen, dtype=torch.float64)
+    v = torch.randn(200, 2, 16, generator=gen, dtype=torch.float64)
+    o, lse = orc.window_attention_ref(q, k, v, cu, 10, dtype=torch.float64)
+    for s0, s1 in ((0, 70), (70, 71), (71, 200)):
+        L = s1 - s0
+        i, p = torch.arange(L)[:, None], torch.arange(L)[None, :]
+        mask = (p <= i) & (p >= i - 10)
+        kx, vx = k[s0:s1].repeat_interleave(2, 1), v[s0:s1].repeat_interleave(2, 1)
+        ref = F.scaled_dot_product_attention(q[s0:s1].transpose(0, 1)[None], kx.transpose(0, 1)[None],
+                                             vx.transpose(0, 1)[None], attn_mask=mask[None, None])[0].transpose(0, 1)
+        assert torch.allclose(o[s0:s1], ref, atol=1e-10)
+    # a window at least as long as the sequence is plain causal attention
+    o2, _ = orc.window_attention_ref(q[:70], k[:70], v[:70], [0, 70], 1000, dtype=torch.float64)
+    kx, vx = k[:70].repeat_interleave(2, 1), v[:70].repeat_interleave(2, 1)
+    ref = F.scaled_dot_product_attention(q[:70].transpose(0, 1)[None], kx.transpose(0, 1)[None],
+                                         vx.transpose(0, 1)[None], is_causal=True)[0].transpose(0, 1)
+    assert torch.allclose(o2, ref, atol=1e-10)
+    # token 0 of every sequence sees itself only
+    assert torch.allclose(o[71], v[71].repeat_interleave(2, 0), atol=1e-12)
+
+
+def test_llama3_inv_freq_against_transformers():
+    inv = orc.llama3_inv_freq(128, 500000.0)
+    assert inv.shape == (64,) and inv.dtype == torch.float32
+    base = 1.0 / (500000.0 ** (torch.arange(0, 128, 2).float() / 128))
+    assert torch.equal(orc.llama3_inv_freq(128, 500000.0, factor=1.0), base)
+    assert torch.equal(inv[:16], base[:16])            # short wavelengths untouched
+    assert torch.allclose(inv[-8:], base[-8:] / 8.0)    # long wavelengths divided by the factor
+    tr = pytest.importorskip("transformers.modeling_rope_utils")
+
+    class Cfg:
+        max_position_embeddings = 131072
+        head_dim = 128
+        rope_theta = 500000.0
+        hidden_size = 4096
+        num_attention_heads = 32
+        partial_rotary_factor = 1.0
+        rope_scaling = {"factor": 8.0, "high_freq_factor": 4.0, "low_freq_factor": 1.0,
+                        "original_max_position_embeddings": 8192, "rope_type": "llama3"}
+        rope_parameters = dict(rope_scaling, rope_theta=500000.0)
+
+        def standardize_rope_params(self):
+            pass
+
+    try:
+        ref, scale = tr.ROPE_INIT_FUNCTIONS["llama3"](Cfg(), "cpu")
+    except Exception as e:  # the installed transformers wants a different config shape
+        pytest.skip(f"transformers rope init not callable with a plain config: {e}")
+    assert scale == 1.0
+    assert torch.allclose(inv, ref.float(), rtol=1e-6, atol=0)
+
+
+def test_rope_invariants():
+    gen = torch.Generator().manual_seed(1)
+    inv = orc.llama3_inv_freq(32, 10000.0, original_max=64)
+    cu = [0, 40, 100]
+    x = torch.randn(100, 2, 32, generator=gen, dtype=torch.float64)
+    y = orc.rope_ref(x, cu, inv)
+    # pairs (d, d + D/2) are rotated: their norm is preserved
+    n_in = x[..., :16] ** 2 + x[..., 16:] ** 2
+    n_out = y[..., :16] ** 2 + y[..., 16:] ** 2
+    assert torch.allclose(n_in.float(), n_out, atol=1e-5)
+    # position 0 is the identity, also at the start of the second sequence
+    assert torch.allclose(y[0], x[0].float(), atol=1e-7) and torch.allclose(y[40], x[40].float(), atol=1e-7)
+    # relative-position property: <rope(a, m), rope(b, n)> depends on m - n only
+    a = torch.randn(1, 1, 32, generator=gen, dtype=torch.float64).expand(60, 1, 32).contiguous()
+    b = torch.randn(1, 1, 32, generator=gen, dtype=torch.float64).expand(60, 1, 32).contiguous()
+    ra, rb = orc.rope_ref(a, [0, 60], inv), orc.rope_ref(b, [0, 60], inv)
+    d1 = (ra[10, 0] * rb[3, 0]).sum()
+    d2 = (ra[47, 0] * rb[40, 0]).sum()
+    assert abs(float(d1 - d2)) < 1e-4
+    # strided positions: token j sits at start + j*stride
+    ys = orc.rope_ref(x[:10], [0, 10], inv, start=0, stride=4)
+    assert torch.allclose(ys[3], orc.rope_ref(x[:40], [0, 40], inv)[12] * 0 + orc.rope_ref(
+        torch.cat([x[:12], x[3:4], x[13:40]]), [0, 40], inv)[12], atol=1e-6)
+    # the conjugate rotation undoes the rotation
+    back = orc.rope_ref(y.double(), cu, inv, conj=True)
+    assert torch.allclose(back, x.float(), atol=1e-5)
