@@ -1,0 +1,418 @@
+// Kernels the attention layer needs around the hot path (gfx950):
+//   rope          : rotary embedding on packed sequences (forward, and its inverse
+//                   rotation = backward), positions start + j*stride per sequence
+//   lc_fwd        : linear compression y[n,h,:] = sum_k x[n*stride+k,h,:] W[h,k] (+ bias)
+//                   as a strided-window GEMM: Y^T = W^T X^T on 32x32x16 MFMA, W tiles
+//                   through LDS with transposing reads, X rows straight from memory
+//   lc_dx / lc_dw : its backward without atomics: dX^T = sum_r W[h,k_r] dY[n_r]^T per
+//                   token phase, and dW[h,k] = X_k^T dY with both operands read
+//                   transposed from LDS tiles
+//
+// Semantics: nsa_ref/module/rope.py:64-134, nsa_ref/ops/linear_compress.py:28-131
+// (forward), :135-292 (backward, fp32 atomics there), :474-502 (positional bias).
+#include "fsa_common.h"
+
+namespace fsa {
+
+// ------------------------------------------------------------------- rope ----
+template <typename T>
+__global__ void __launch_bounds__(256)
+rope_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, T* __restrict__ out, int64_t o_sn,
+            int64_t o_sh, const int32_t* __restrict__ cu, int batch, int64_t n, int h, int d,
+            const float* __restrict__ inv_freq, float attn_scale, int start, int stride, int conj) {
+  typedef typename Elem<T>::vec8 vec8;
+  const int lpr = d / 16;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = idx / lpr;
+  const int sub = (int)(idx - row * lpr);
+  if (row >= n * h) return;
+  const int64_t tok = row / h;
+  const int head = (int)(row - tok * h);
+  const int s = upper_seg(cu, batch, (int)tok);
+  const float pos = (float)(start + ((int)tok - cu[s]) * stride);
+  const T* xr = x + tok * x_sn + (int64_t)head * x_sh + sub * 8;
+  vec8 a = load16<vec8>(xr), b = load16<vec8>(xr + d / 2);
+  vec8 oa, ob;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float ang = pos * inv_freq[sub * 8 + e];
+    // the tables are rounded to the tensor's dtype before use, as in the reference
+    const float c = (float)(T)(cosf(ang) * attn_scale);
+    float sn = (float)(T)(sinf(ang) * attn_scale);
+    if (conj) sn = -sn;
+    const float x1 = (float)a[e], x2 = (float)b[e];
+    oa[e] = (T)(x1 * c - x2 * sn);
+    ob[e] = (T)(x1 * sn + x2 * c);
+  }
+  T* orow = out + tok * o_sn + (int64_t)head * o_sh + sub * 8;
+  store16(orow, oa);
+  store16(orow + d / 2, ob);
+}
+
+// ------------------------------------------------------- linear compress ----
+constexpr int LC_KC = 64;     // contraction chunk staged per step
+constexpr int LC_ROWS = 128;  // compressed tokens (or tokens) per work-group
+
+// transposing read of 8 consecutive rows r0..r0+7 of one column out of a row-major LDS tile:
+// this lane supplies the address of row r0 + (lane%16)/4, columns c0 + 4*(lane%4)
+template <typename T>
+__device__ __forceinline__ typename Elem<T>::vec8 lds_tr8_rows(const T* p, int stride) {
+  typename Elem<T>::vec4 lo = lds_read_tr4<T>(p);
+  typename Elem<T>::vec4 hi = lds_read_tr4<T>(p + 4 * stride);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+template <typename T, int D>
+__global__ void __launch_bounds__(256)
+lc_fwd_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __restrict__ w,
+              const T* __restrict__ bias, T* __restrict__ y, const int32_t* __restrict__ cu_x,
+              const int32_t* __restrict__ cu_y, int nheads, int ks, int stride) {
+  typedef typename Elem<T>::vec8 vec8;
+  typedef typename Elem<T>::vec4 vec4;
+  constexpr int WS = D + 8, NT = D / 32;
+  __shared__ __attribute__((aligned(16))) T Wt[LC_KC * WS];
+  const int s = blockIdx.y, h = blockIdx.z;
+  const int y0 = cu_y[s], ny = cu_y[s + 1] - y0, x0 = cu_x[s];
+  const int n_lo = blockIdx.x * LC_ROWS;
+  if (n_lo >= ny) return;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int col = lane & 31, hh = lane >> 5;
+  const int n = n_lo + wv * 32 + col;
+  const bool valid = n < ny;
+  const T* xrow0 = x + (int64_t)(x0 + (valid ? n : 0) * stride) * x_sn + (int64_t)h * x_sh + 8 * hh;
+  const T* wh = w + (int64_t)h * ks * D * D;
+  const int tr_row = (lane & 15) >> 2, tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  f32x16 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+  for (int k = 0; k < ks; ++k)
+    for (int dc = 0; dc < D; dc += LC_KC) {
+      __syncthreads();
+      for (int c = tid; c < LC_KC * (D / 8); c += 256) {
+        const int r = c / (D / 8), cc = c % (D / 8);
+        store16(&Wt[r * WS + cc * 8], load16<vec8>(wh + ((int64_t)k * D + dc + r) * D + cc * 8));
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < LC_KC / 16; ++kk) {
+        vec8 xf = zero8<T>();
+        if (valid) xf = load16<vec8>(xrow0 + (int64_t)k * x_sn + dc + 16 * kk);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          vec8 wf = lds_tr8_rows<T>(&Wt[(16 * kk + 8 * hh + tr_row) * WS + t * 32 + tr_col], WS);
+          acc[t] = Elem<T>::mfma32(wf, xf, acc[t]);
+        }
+      }
+    }
+  if (!valid) return;
+  T* yrow = y + ((int64_t)(y0 + n) * nheads + h) * D + 4 * hh;
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      vec4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        T r = (T)acc[t][4 * qd + e];
+        if (bias) r = (T)((float)r + (float)bias[h * D + t * 32 + 8 * qd + 4 * hh + e]);
+        v[e] = r;
+      }
+      store8(yrow + t * 32 + 8 * qd, v);
+    }
+}
+
+// bias[h, dout] = sum_{k,d} pe[h,k,d] W[h,k,d,dout]  (fp32 accumulation, rounded once)
+template <typename T>
+__global__ void __launch_bounds__(256)
+lc_bias_kernel(const T* __restrict__ pe, const T* __restrict__ w, T* __restrict__ bias, int kd, int d) {
+  __shared__ float part[256];
+  const int h = blockIdx.x, tid = threadIdx.x;
+  const int dout = tid % d, slice = tid / d, nslice = 256 / d;
+  float s = 0.f;
+  for (int i = slice; i < kd; i += nslice) s += (float)pe[(int64_t)h * kd + i] * (float)w[((int64_t)h * kd + i) * d + dout];
+  part[tid] = s;
+  __syncthreads();
+  if (slice == 0) {
+    for (int j = 1; j < nslice; ++j) s += part[j * d + dout];
+    bias[h * d + dout] = (T)s;
+  }
+}
+
+// dX: one wave = 32 tokens of one phase (t % stride), so that the window offsets k_r are wave-uniform
+template <typename T, int D>
+__global__ void __launch_bounds__(256)
+lc_dx_kernel(const T* __restrict__ dy, const T* __restrict__ w, T* __restrict__ dx,
+             const int32_t* __restrict__ cu_x, const int32_t* __restrict__ cu_y, int nheads, int ks,
+             int stride) {
+  typedef typename Elem<T>::vec8 vec8;
+  typedef typename Elem<T>::vec4 vec4;
+  constexpr int NT = D / 32;
+  const int s = blockIdx.y, h = blockIdx.z;
+  const int x0 = cu_x[s], len = cu_x[s + 1] - x0, y0 = cu_y[s], ny = cu_y[s + 1] - y0;
+  const int m_per_phase = (len + stride - 1) / stride;
+  const int tiles_per_phase = (m_per_phase + LC_ROWS - 1) / LC_ROWS;
+  const int phase = blockIdx.x / tiles_per_phase, mt = blockIdx.x % tiles_per_phase;
+  if (phase >= stride || len == 0) return;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int col = lane & 31, hh = lane >> 5;
+  const int m = mt * LC_ROWS + wv * 32 + col;
+  const int t = phase + stride * m;
+  const bool valid = t < len;
+  const int nrep = ks / stride;
+  f32x16 acc[NT];
+#pragma unroll
+  for (int i_ = 0; i_ < NT; ++i_)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i_][i] = 0.f;
+  for (int r = 0; r < nrep; ++r) {
+    const int nwin = m - r, k = phase + r * stride;
+    const bool ok = valid && nwin >= 0 && nwin < ny;
+    const T* dyrow = dy + ((int64_t)(y0 + (ok ? nwin : 0)) * nheads + h) * D + 8 * hh;
+    const T* wk = w + ((int64_t)h * ks + k) * D * D + 8 * hh;
+#pragma unroll
+    for (int kk = 0; kk < D / 16; ++kk) {
+      vec8 yf = zero8<T>();
+      if (ok) yf = load16<vec8>(dyrow + 16 * kk);
+#pragma unroll
+      for (int i_ = 0; i_ < NT; ++i_) {
+        vec8 wf = load16<vec8>(wk + (int64_t)(i_ * 32 + col) * D + 16 * kk);  // A[m = d][k = dout]
+        acc[i_] = Elem<T>::mfma32(wf, yf, acc[i_]);
+      }
+    }
+  }
+  if (!valid) return;
+  T* xrow = dx + ((int64_t)(x0 + t) * nheads + h) * D + 4 * hh;
+#pragma unroll
+  for (int i_ = 0; i_ < NT; ++i_)
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      vec4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = (T)acc[i_][4 * qd + e];
+      store8(xrow + i_ * 32 + 8 * qd, v);
+    }
+}
+
+// dbias[h, dout] = sum_n dY[n, h, dout]  (fp32)
+template <typename T>
+__global__ void __launch_bounds__(256)
+lc_dbias_kernel(const T* __restrict__ dy, float* __restrict__ dbias, int64_t ny_total, int nheads, int d) {
+  __shared__ float part[256];
+  const int h = blockIdx.x, tid = threadIdx.x;
+  const int dout = tid % d, slice = tid / d, nslice = 256 / d;
+  float s = 0.f;
+  for (int64_t n = slice; n < ny_total; n += nslice) s += (float)dy[(n * nheads + h) * d + dout];
+  part[tid] = s;
+  __syncthreads();
+  if (slice == 0) {
+    for (int j = 1; j < nslice; ++j) s += part[j * d + dout];
+    dbias[h * d + dout] = s;
+  }
+}
+
+// dpe[h, k, d] = sum_dout W[h,k,d,dout] dbias[h,dout]
+template <typename T>
+__global__ void __launch_bounds__(256)
+lc_dpe_kernel(const T* __restrict__ w, const float* __restrict__ dbias, T* __restrict__ dpe, int kd, int d) {
+  const int h = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= kd) return;
+  const T* wr = w + ((int64_t)h * kd + i) * d;
+  float s = 0.f;
+  for (int o = 0; o < d; ++o) s += (float)wr[o] * dbias[h * d + o];
+  dpe[(int64_t)h * kd + i] = (T)s;
+}
+
+// dW[h, k, d, dout] = sum_n x[tok(n) + k, h, d] dY[n, h, dout] (+ pe[h,k,d] dbias[h,dout])
+template <typename T, int D>
+__global__ void __launch_bounds__(256)
+lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __restrict__ dy,
+             const T* __restrict__ pe, const float* __restrict__ dbias, T* __restrict__ dw,
+             const int32_t* __restrict__ cu_x, const int32_t* __restrict__ cu_y, int batch, int nheads,
+             int ks, int stride) {
+  typedef typename Elem<T>::vec8 vec8;
+  constexpr int XS = 128 + 8, YS = D + 8, NT = D / 32;
+  __shared__ __attribute__((aligned(16))) T Xs[LC_KC * XS];
+  __shared__ __attribute__((aligned(16))) T Ys[LC_KC * YS];
+  const int k = blockIdx.x, h = blockIdx.y, dz = blockIdx.z * 128;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int col = lane & 31, hh = lane >> 5;
+  const int ny_total = cu_y[batch];
+  const int tr_row = (lane & 15) >> 2, tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  f32x16 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+  for (int n0 = 0; n0 < ny_total; n0 += LC_KC) {
+    __syncthreads();
+    for (int c = tid; c < LC_KC * 16; c += 256) {  // X rows: 128 dims = 16 chunks
+      const int r = c / 16, cc = c % 16;
+      const int n = n0 + r;
+      vec8 v = zero8<T>();
+      if (n < ny_total) {
+        const int s = upper_seg(cu_y, batch, n);
+        const int64_t tok = cu_x[s] + (int64_t)(n - cu_y[s]) * stride + k;
+        v = load16<vec8>(x + tok * x_sn + (int64_t)h * x_sh + dz + cc * 8);
+      }
+      store16(&Xs[r * XS + cc * 8], v);
+    }
+    for (int c = tid; c < LC_KC * (D / 8); c += 256) {
+      const int r = c / (D / 8), cc = c % (D / 8);
+      const int n = n0 + r;
+      vec8 v = zero8<T>();
+      if (n < ny_total) v = load16<vec8>(dy + ((int64_t)n * nheads + h) * D + cc * 8);
+      store16(&Ys[r * YS + cc * 8], v);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < LC_KC / 16; ++kk) {
+      vec8 xf = lds_tr8_rows<T>(&Xs[(16 * kk + 8 * hh + tr_row) * XS + wv * 32 + tr_col], XS);  // A[m = d][k = n]
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        vec8 yf = lds_tr8_rows<T>(&Ys[(16 * kk + 8 * hh + tr_row) * YS + t * 32 + tr_col], YS);  // B[k = n][dout]
+        acc[t] = Elem<T>::mfma32(xf, yf, acc[t]);
+      }
+    }
+  }
+  // C layout: lane column = dout within the tile, registers = d rows
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int dd = dz + wv * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+      const int dout = t * 32 + col;
+      float v = acc[t][i];
+      if (pe) v += (float)pe[((int64_t)h * ks + k) * D + dd] * dbias[h * D + dout];
+      dw[(((int64_t)h * ks + k) * D + dd) * D + dout] = (T)v;
+    }
+}
+
+}  // namespace fsa
+
+using namespace fsa;
+
+extern "C" int fsa_rope(const void* x, void* out, int32_t dtype, int64_t x_stride_n, int64_t x_stride_h,
+                        int64_t o_stride_n, int64_t o_stride_h, const int32_t* cu_seqlens, int32_t batch,
+                        int64_t total_tokens, int32_t num_heads, int32_t head_dim, const float* inv_freq,
+                        float attention_scaling, int32_t start, int32_t stride, int32_t inverse,
+                        void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FSA_CHECK_ARG(x && out && cu_seqlens && inv_freq, "fsa_rope: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_rope: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(head_dim >= 16 && head_dim % 16 == 0, "fsa_rope: head_dim must be a multiple of 16");
+  FSA_CHECK_ARG(batch >= 1 && num_heads >= 1, "fsa_rope: bad sizes");
+  if (total_tokens == 0) return 0;
+  const int64_t work = total_tokens * num_heads * (head_dim / 16);
+  const unsigned grid = (unsigned)((work + 255) / 256);
+  ProfScope ps_("rope", stream);
+  if (dtype == FSA_BF16)
+    rope_kernel<__bf16><<<grid, 256, 0, stream>>>((const __bf16*)x, x_stride_n, x_stride_h, (__bf16*)out,
+                                                  o_stride_n, o_stride_h, cu_seqlens, batch, total_tokens,
+                                                  num_heads, head_dim, inv_freq, attention_scaling, start,
+                                                  stride, inverse);
+  else
+    rope_kernel<_Float16><<<grid, 256, 0, stream>>>((const _Float16*)x, x_stride_n, x_stride_h, (_Float16*)out,
+                                                    o_stride_n, o_stride_h, cu_seqlens, batch, total_tokens,
+                                                    num_heads, head_dim, inv_freq, attention_scaling, start,
+                                                    stride, inverse);
+  FSA_CHECK_LAUNCH("fsa_rope");
+  return 0;
+}
+
+template <typename T>
+static int lc_fwd_t(const void* x, int64_t x_sn, int64_t x_sh, const void* w, const void* pe, void* bias,
+                    void* y, const int32_t* cu_x, const int32_t* cu_y, int batch, int64_t max_y, int h, int d,
+                    int ks, int stride, hipStream_t stream) {
+  if (pe) {
+    ProfScope ps_("linear_compress_bias", stream);
+    lc_bias_kernel<T><<<h, 256, 0, stream>>>((const T*)pe, (const T*)w, (T*)bias, ks * d, d);
+  }
+  dim3 grid((unsigned)((max_y + LC_ROWS - 1) / LC_ROWS), batch, h);
+  ProfScope ps_("linear_compress_fwd", stream);
+  const T* b = pe ? (const T*)bias : nullptr;
+  if (d == 64) lc_fwd_kernel<T, 64><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)w, b, (T*)y, cu_x, cu_y, h, ks, stride);
+  else if (d == 128) lc_fwd_kernel<T, 128><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)w, b, (T*)y, cu_x, cu_y, h, ks, stride);
+  else lc_fwd_kernel<T, 256><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)w, b, (T*)y, cu_x, cu_y, h, ks, stride);
+  return 0;
+}
+
+extern "C" int fsa_linear_compress_fwd(const void* x, const void* w, const void* pe, int32_t dtype,
+                                       int64_t x_stride_n, int64_t x_stride_h, const int32_t* cu_seqlens_x,
+                                       const int32_t* cu_seqlens_y, int32_t batch, int64_t max_seqlen_y,
+                                       int32_t num_heads, int32_t head_dim, int32_t kernel_size,
+                                       int32_t kernel_stride, void* y, void* bias_scratch, void* stream_) {
+  FSA_CHECK_ARG(x && w && y && cu_seqlens_x && cu_seqlens_y, "fsa_linear_compress_fwd: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_linear_compress_fwd: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(head_dim == 64 || head_dim == 128 || head_dim == 256,
+                "fsa_linear_compress_fwd: head_dim=%d not supported (64, 128, 256)", head_dim);
+  FSA_CHECK_ARG(kernel_stride >= 1 && kernel_size % kernel_stride == 0,
+                "fsa_linear_compress_fwd: kernel_size must be a multiple of kernel_stride");
+  FSA_CHECK_ARG(!pe || bias_scratch, "fsa_linear_compress_fwd: bias scratch [H, D] needed with pe");
+  if (max_seqlen_y <= 0) return 0;
+  hipStream_t stream = (hipStream_t)stream_;
+  if (dtype == FSA_BF16)
+    lc_fwd_t<__bf16>(x, x_stride_n, x_stride_h, w, pe, bias_scratch, y, cu_seqlens_x, cu_seqlens_y, batch,
+                     max_seqlen_y, num_heads, head_dim, kernel_size, kernel_stride, stream);
+  else
+    lc_fwd_t<_Float16>(x, x_stride_n, x_stride_h, w, pe, bias_scratch, y, cu_seqlens_x, cu_seqlens_y, batch,
+                       max_seqlen_y, num_heads, head_dim, kernel_size, kernel_stride, stream);
+  FSA_CHECK_LAUNCH("fsa_linear_compress_fwd");
+  return 0;
+}
+
+template <typename T>
+static int lc_bwd_t(const void* x, int64_t x_sn, int64_t x_sh, const void* w, const void* pe, const void* dy,
+                    const int32_t* cu_x, const int32_t* cu_y, int batch, int64_t max_x, int64_t total_y, int h,
+                    int d, int ks, int stride, void* dx, void* dw, void* dpe, float* dbias, hipStream_t stream) {
+  {
+    ProfScope ps_("linear_compress_dx", stream);
+    const int64_t m_per_phase = (max_x + stride - 1) / stride;
+    dim3 grid((unsigned)(stride * ((m_per_phase + LC_ROWS - 1) / LC_ROWS)), batch, h);
+    // the grid is sized for the longest sequence; shorter sequences recompute their own tiling inside
+    if (d == 64) lc_dx_kernel<T, 64><<<grid, 256, 0, stream>>>((const T*)dy, (const T*)w, (T*)dx, cu_x, cu_y, h, ks, stride);
+    else if (d == 128) lc_dx_kernel<T, 128><<<grid, 256, 0, stream>>>((const T*)dy, (const T*)w, (T*)dx, cu_x, cu_y, h, ks, stride);
+    else lc_dx_kernel<T, 256><<<grid, 256, 0, stream>>>((const T*)dy, (const T*)w, (T*)dx, cu_x, cu_y, h, ks, stride);
+  }
+  if (pe) {
+    ProfScope ps_("linear_compress_dbias", stream);
+    lc_dbias_kernel<T><<<h, 256, 0, stream>>>((const T*)dy, dbias, total_y, h, d);
+    lc_dpe_kernel<T><<<dim3((ks * d + 255) / 256, h), 256, 0, stream>>>((const T*)w, dbias, (T*)dpe, ks * d, d);
+  }
+  {
+    ProfScope ps_("linear_compress_dw", stream);
+    dim3 grid(ks, h, d / 128 > 0 ? d / 128 : 1);
+    const T* pe_ = (const T*)pe;
+    if (d == 128) lc_dw_kernel<T, 128><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)dy, pe_, dbias, (T*)dw, cu_x, cu_y, batch, h, ks, stride);
+    else lc_dw_kernel<T, 256><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)dy, pe_, dbias, (T*)dw, cu_x, cu_y, batch, h, ks, stride);
+  }
+  return 0;
+}
+
+extern "C" int fsa_linear_compress_bwd(const void* x, const void* w, const void* pe, const void* dy,
+                                       int32_t dtype, int64_t x_stride_n, int64_t x_stride_h,
+                                       const int32_t* cu_seqlens_x, const int32_t* cu_seqlens_y,
+                                       int32_t batch, int64_t max_seqlen_x, int64_t total_y,
+                                       int32_t num_heads, int32_t head_dim, int32_t kernel_size,
+                                       int32_t kernel_stride, void* dx, void* dw, void* dpe,
+                                       float* dbias_scratch, void* stream_) {
+  FSA_CHECK_ARG(x && w && dy && dx && dw && cu_seqlens_x && cu_seqlens_y, "fsa_linear_compress_bwd: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_linear_compress_bwd: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(head_dim == 128 || head_dim == 256,
+                "fsa_linear_compress_bwd: head_dim=%d not supported (128, 256)", head_dim);
+  FSA_CHECK_ARG(kernel_stride >= 1 && kernel_size % kernel_stride == 0,
+                "fsa_linear_compress_bwd: kernel_size must be a multiple of kernel_stride");
+  FSA_CHECK_ARG(!pe || (dpe && dbias_scratch), "fsa_linear_compress_bwd: dpe and dbias scratch needed with pe");
+  FSA_CHECK_ARG(max_seqlen_x >= 1, "fsa_linear_compress_bwd: bad max_seqlen_x");
+  hipStream_t stream = (hipStream_t)stream_;
+  if (dtype == FSA_BF16)
+    lc_bwd_t<__bf16>(x, x_stride_n, x_stride_h, w, pe, dy, cu_seqlens_x, cu_seqlens_y, batch, max_seqlen_x, total_y,
+                     num_heads, head_dim, kernel_size, kernel_stride, dx, dw, dpe, dbias_scratch, stream);
+  else
+    lc_bwd_t<_Float16>(x, x_stride_n, x_stride_h, w, pe, dy, cu_seqlens_x, cu_seqlens_y, batch, max_seqlen_x,
+                       total_y, num_heads, head_dim, kernel_size, kernel_stride, dx, dw, dpe, dbias_scratch, stream);
+  FSA_CHECK_LAUNCH("fsa_linear_compress_bwd");
+  return 0;
+}

@@ -57,6 +57,11 @@ SIGNATURES = {
                                   i64, i64, i64, i64, i64, i64, i64, i64, i64, i64,
                                   vp, i32, i64, i64, i32, i32, i32, i32, f32,
                                   vp, vp, vp, vp, sz, vp]),
+    "fsa_rope": (C.c_int, [vp, vp, i32, i64, i64, i64, i64, vp, i32, i64, i32, i32, vp, f32, i32, i32, i32, vp]),
+    "fsa_linear_compress_fwd": (C.c_int, [vp, vp, vp, i32, i64, i64, vp, vp, i32, i64, i32, i32, i32, i32,
+                                          vp, vp, vp]),
+    "fsa_linear_compress_bwd": (C.c_int, [vp, vp, vp, vp, i32, i64, i64, vp, vp, i32, i64, i64, i32, i32,
+                                          i32, i32, vp, vp, vp, vp, vp]),
     "fsa_decode_cmpattn": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp,
                                      i32, i32, i32, i32, i32, i32, f32, i32, vp, vp, vp, i64, vp]),
     "fsa_decode_topk": (C.c_int, [vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,

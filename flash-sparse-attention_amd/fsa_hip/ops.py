@@ -343,3 +343,57 @@ def winattn_bwd(q, k, v, o, do, lse, cu_seqlens, max_seqlen, window, softmax_sca
                              _ptr(dv), _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_winattn_bwd")
     return dq, dk, dv
+
+
+def rope(x, cu_seqlens, inv_freq, attention_scaling=1.0, start=0, stride=1, inverse=False):
+    """Rotary embedding on packed sequences; inverse=True is the backward rotation."""
+    _require_cuda(x, cu_seqlens, inv_freq)
+    assert x.dtype in _DTYPE and x.dim() == 3 and x.stride(2) == 1
+    assert inv_freq.dtype == torch.float32 and inv_freq.numel() == x.shape[2] // 2
+    lib = _lib.load()
+    n, h, d = x.shape
+    out = torch.empty((n, h, d), dtype=x.dtype, device=x.device)
+    rc = lib.fsa_rope(_ptr(x), _ptr(out), _DTYPE[x.dtype], x.stride(0), x.stride(1), out.stride(0), out.stride(1),
+                      _ptr(cu_seqlens), cu_seqlens.numel() - 1, n, h, d, _ptr(inv_freq.contiguous()),
+                      float(attention_scaling), int(start), int(stride), 1 if inverse else 0, _stream(x.device))
+    _lib.check(rc, "fsa_rope")
+    return out
+
+
+def linear_compress_fwd(x, w, cu_x, cu_y, total_y, max_y, kernel_size, kernel_stride, pe=None):
+    """y [total_y, H, D] = strided-window projection of x [N, H, D] with w [H, ks*D, D] (+ pe bias)."""
+    _require_cuda(x, w, cu_x, cu_y)
+    assert x.dtype in _DTYPE and x.dtype == w.dtype and x.stride(2) == 1 and w.is_contiguous()
+    lib = _lib.load()
+    n, h, d = x.shape
+    y = torch.empty((int(total_y), h, d), dtype=x.dtype, device=x.device)
+    bias = torch.empty((h, d), dtype=x.dtype, device=x.device) if pe is not None else None
+    if pe is not None:
+        assert pe.dtype == x.dtype and pe.is_contiguous()
+    if total_y > 0:
+        rc = lib.fsa_linear_compress_fwd(_ptr(x), _ptr(w), _ptr(pe), _DTYPE[x.dtype], x.stride(0), x.stride(1),
+                                         _ptr(cu_x), _ptr(cu_y), cu_x.numel() - 1, int(max_y), h, d, kernel_size,
+                                         kernel_stride, _ptr(y), _ptr(bias), _stream(x.device))
+        _lib.check(rc, "fsa_linear_compress_fwd")
+    return y
+
+
+def linear_compress_bwd(x, w, dy, cu_x, cu_y, max_x, kernel_size, kernel_stride, pe=None):
+    """(dx, dw, dpe or None) of linear_compress_fwd."""
+    _require_cuda(x, w, dy, cu_x, cu_y)
+    lib = _lib.load()
+    n, h, d = x.shape
+    dev = x.device
+    dy = dy.contiguous()
+    dx = torch.empty((n, h, d), dtype=x.dtype, device=dev)
+    dw = torch.empty_like(w)
+    dpe = torch.empty_like(pe) if pe is not None else None
+    dbias = torch.empty((h, d), dtype=torch.float32, device=dev) if pe is not None else None
+    if dy.shape[0] == 0:
+        return dx.zero_(), dw.zero_(), (dpe.zero_() if dpe is not None else None)
+    rc = lib.fsa_linear_compress_bwd(_ptr(x), _ptr(w), _ptr(pe), _ptr(dy), _DTYPE[x.dtype], x.stride(0),
+                                     x.stride(1), _ptr(cu_x), _ptr(cu_y), cu_x.numel() - 1, int(max_x),
+                                     dy.shape[0], h, d, kernel_size, kernel_stride, _ptr(dx), _ptr(dw), _ptr(dpe),
+                                     _ptr(dbias), _stream(dev))
+    _lib.check(rc, "fsa_linear_compress_bwd")
+    return dx, dw, dpe

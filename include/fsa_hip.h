@@ -276,6 +276,42 @@ int fsa_winattn_bwd(const void* q, const void* k, const void* v, const void* o, 
                     float softmax_scale, void* dq, void* dk, void* dv, void* workspace,
                     size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Rotary embedding on packed sequences (non-interleaved halves): token j of a
+ * sequence sits at position start + j*stride; cos/sin are evaluated in fp32 from
+ * inv_freq [D/2] (device), scaled by attention_scaling and rounded to the tensor
+ * dtype before the fp32 rotation.  inverse != 0 applies the opposite rotation,
+ * which is the backward of the forward.  Replaces RotaryEmbedding.forward /
+ * flash_attn apply_rotary_emb (nsa_ref/module/rope.py:89-134).
+ * ---------------------------------------------------------------------- */
+int fsa_rope(const void* x, void* out, int32_t dtype, int64_t x_stride_n, int64_t x_stride_h,
+             int64_t o_stride_n, int64_t o_stride_h, const int32_t* cu_seqlens, int32_t batch,
+             int64_t total_tokens, int32_t num_heads, int32_t head_dim, const float* inv_freq,
+             float attention_scaling, int32_t start, int32_t stride, int32_t inverse, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Linear compression of keys / values:
+ *   y[n, h, :] = sum_{k < kernel_size} x[n*kernel_stride + k, h, :] @ W[h, k]   (+ pe-bias)
+ * with W = w viewed as [H, kernel_size, D, D], y_len = floor((len - ks)/stride) + 1
+ * (0 if len < ks), cu_seqlens_y given by the caller.  pe [H, ks, D] is optional;
+ * its contribution einsum(pe, W) is rounded to the dtype and added to the rounded
+ * y, as in the reference.  Replaces linear_compress / LinearCompress and their
+ * kernels (nsa_ref/ops/linear_compress.py:28-131, 135-292, 295-502); the backward
+ * uses no atomics.  y / dx / dw / dpe are contiguous; bias_scratch is [H, D] of
+ * the dtype, dbias_scratch [H, D] fp32.
+ * ---------------------------------------------------------------------- */
+int fsa_linear_compress_fwd(const void* x, const void* w, const void* pe, int32_t dtype,
+                            int64_t x_stride_n, int64_t x_stride_h, const int32_t* cu_seqlens_x,
+                            const int32_t* cu_seqlens_y, int32_t batch, int64_t max_seqlen_y,
+                            int32_t num_heads, int32_t head_dim, int32_t kernel_size, int32_t kernel_stride,
+                            void* y, void* bias_scratch, void* stream);
+
+int fsa_linear_compress_bwd(const void* x, const void* w, const void* pe, const void* dy, int32_t dtype,
+                            int64_t x_stride_n, int64_t x_stride_h, const int32_t* cu_seqlens_x,
+                            const int32_t* cu_seqlens_y, int32_t batch, int64_t max_seqlen_x, int64_t total_y,
+                            int32_t num_heads, int32_t head_dim, int32_t kernel_size, int32_t kernel_stride,
+                            void* dx, void* dw, void* dpe, float* dbias_scratch, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

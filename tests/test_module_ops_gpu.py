@@ -1,0 +1,80 @@
+"""GPU parity: rotary embedding and linear compression (forward / backward) vs the CPU oracle."""
+import math
+
+import pytest
+import torch
+
+from fsa_hip import ops
+from oracle import cmpattn as pre
+from oracle import module as orc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("start,stride", [(0, 1), (0, 16)])
+def test_rope(dev, dtype, start, stride):
+    gen = torch.Generator().manual_seed(41)
+    cu = [0, 1000, 1001, 3000]
+    x = torch.randn(3000, 6, 128, generator=gen).to(dtype)
+    inv = orc.llama3_inv_freq(128, 500000.0)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    y = ops.rope(x.to(dev), cu_t, inv.to(dev), 1.0, start, stride)
+    back = ops.rope(y, cu_t, inv.to(dev), 1.0, start, stride, inverse=True)
+    torch.cuda.synchronize()
+    ref = orc.rope_ref(x, cu, inv, start, stride, table_dtype=dtype)
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    # identical arithmetic up to the rounding of cos/sin (one table ulp on a few entries) and of the output
+    err = (y.float().cpu() - ref).abs()
+    assert (err <= 3 * ulp * ref.abs() + 4 * ulp).all(), err.max()
+    assert (err > ulp * ref.abs() + 1e-6).float().mean().item() < 0.02
+    err_b = (back.float().cpu() - x.float()).abs().max().item()
+    assert err_b <= 8 * ulp * 4
+
+
+CASES = [
+    # cu_seqlens, H, D, ks, stride, dtype, with pe
+    ([0, 2048], 4, 128, 32, 16, torch.bfloat16, True),
+    ([0, 20, 700, 731, 2100, 3000], 2, 128, 32, 16, torch.bfloat16, True),
+    ([0, 1500], 2, 128, 32, 16, torch.float16, False),
+    ([0, 1100], 2, 256, 32, 16, torch.float16, True),
+]
+
+
+@pytest.mark.parametrize("cu,h,d,ks,st,dtype,with_pe", CASES)
+def test_linear_compress_fwd_bwd(dev, cu, h, d, ks, st, dtype, with_pe):
+    print(f"case cu={cu} h={h} d={d} {dtype} pe={with_pe}", flush=True)
+    gen = torch.Generator().manual_seed(43)
+    n = cu[-1]
+    x = torch.randn(n, h, d, generator=gen).to(dtype)
+    w = (torch.randn(h, ks * d, d, generator=gen) * math.sqrt(6.0 / (ks * d + d))).to(dtype)
+    pe = (torch.randn(h, ks, d, generator=gen) * 0.1).to(dtype) if with_pe else None
+    cu_y = pre.compressed_lens(cu, ks, st)
+    dy = torch.randn(cu_y[-1], h, d, generator=gen).to(dtype)
+    cu_x_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    cu_y_t = torch.tensor(cu_y, dtype=torch.int32, device=dev)
+    max_x = max(b - a for a, b in zip(cu[:-1], cu[1:]))
+    max_y = max(b - a for a, b in zip(cu_y[:-1], cu_y[1:]))
+    xd, wd, dyd = x.to(dev), w.to(dev), dy.to(dev)
+    ped = pe.to(dev) if with_pe else None
+    y = ops.linear_compress_fwd(xd, wd, cu_x_t, cu_y_t, cu_y[-1], max_y, ks, st, ped)
+    dx, dw, dpe = ops.linear_compress_bwd(xd, wd, dyd, cu_x_t, cu_y_t, max_x, ks, st, ped)
+    torch.cuda.synchronize()
+    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    per = pe.float().requires_grad_(True) if with_pe else None
+    y_r, cu_y_r = pre.linear_compress_ref(xr, wr, cu, ks, st, per)
+    assert cu_y_r == cu_y
+    (y_r * dy.float()).sum().backward()
+    pairs = [("y", y, y_r.detach()), ("dx", dx, xr.grad), ("dw", dw, wr.grad)]
+    if with_pe:
+        pairs.append(("dpe", dpe, per.grad))
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    for name, got, ref in pairs:
+        got = got.float().cpu()
+        assert torch.isfinite(got).all(), name
+        rel = ((got - ref).norm() / ref.norm()).item()
+        excess = ((got - ref).abs() - 2 * ulp * ref.abs()).max().item()
+        print(f"  {name}: rel Frobenius {rel:.2e}, max abs {(got - ref).abs().max().item():.3e} "
+              f"(ref max {ref.abs().max().item():.2f})", flush=True)
+        assert rel < 3 * ulp, name
+        assert excess <= (2e-2 if dtype == torch.bfloat16 else 5e-3), name
