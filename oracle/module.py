@@ -94,3 +94,49 @@ def rope_ref(x, cu_seqlens, inv_freq, start: int = 0, stride: int = 1, table_dty
         out[s0:s1, :, : D // 2] = x1 * cos[:, None] - x2 * sin[:, None]
         out[s0:s1, :, D // 2:] = x1 * sin[:, None] + x2 * cos[:, None]
     return out
+
+
+def fsa_layer_ref(params: dict, x, cu_seqlens, cfg: dict, topk_idx=None, table_dtype=None):
+    """fp32 composition of the layer (fsa/module/fsa.py:71-173).  `params` holds the reference's
+    parameter names; `cfg` the constructor arguments plus "inv_freq".  When `topk_idx` is given it
+    replaces the selection computed from the compressed branch (the selection is discrete, so a
+    like-for-like comparison passes the ids the device chose).  Returns (y, topk_idx, parts)."""
+    hq, hkv, d = cfg["num_q_heads"], cfg["num_kv_heads"], cfg["head_dim"]
+    ks, st, bk, t = cfg["kernel_size"], cfg["kernel_stride"], cfg["block_size"], cfg["topk"]
+    xf = x.float()
+    q = (xf @ params["proj_q.weight"].float().t()).view(-1, hq, d)
+    k = (xf @ params["proj_k.weight"].float().t()).view(-1, hkv, d)
+    v = (xf @ params["proj_v.weight"].float().t()).view(-1, hkv, d)
+    ck, cu_k = _cmp.linear_compress_ref(k, params["compress_key"].float(), cu_seqlens, ks, st,
+                                        params["intra_block_pe"].float())
+    cv, _ = _cmp.linear_compress_ref(v, params["compress_value"].float(), cu_seqlens, ks, st, None)
+    inv = cfg["inv_freq"]
+
+    def rope(z, cu, start=0, stride=1):
+        # differentiable rotation (rope_ref writes in place, so restate it functionally here)
+        outs = []
+        for (s0, s1) in _bounds(cu):
+            pos = (start + torch.arange(s1 - s0) * stride).float()
+            ang = pos[:, None] * inv.float()[None, :]
+            cos, sin = ang.cos(), ang.sin()
+            if table_dtype is not None:
+                cos, sin = cos.to(table_dtype).float(), sin.to(table_dtype).float()
+            z1, z2 = z[s0:s1, :, : d // 2], z[s0:s1, :, d // 2:]
+            outs.append(torch.cat([z1 * cos[:, None] - z2 * sin[:, None], z1 * sin[:, None] + z2 * cos[:, None]], -1))
+        return torch.cat(outs, 0) if outs else z
+
+    q = rope(q, cu_seqlens)
+    ck = rope(ck, cu_k, 0, st)
+    o_cmp, lse_cmp = _cmp.compressed_attention_ref(q, ck, cv, ks, st, cu_seqlens, cu_k)
+    if topk_idx is None:
+        max_q = max(b - a for a, b in _bounds(cu_seqlens))
+        topk_idx, _ = _cmp.compressed_topk_ref(q.detach(), ck.detach(), lse_cmp.detach(), ks, st, bk, t, cu_seqlens,
+                                               cu_k, init_blocks=cfg["init_blocks"],
+                                               local_blocks=cfg["local_blocks"], max_seqlen_q=max_q)
+    k = rope(k, cu_seqlens)
+    o_sel, _ = _sel.selected_attention_ref(q, k, v, topk_idx, bk, cu_seqlens)
+    o_win, _ = window_attention_ref(q, k, v, cu_seqlens, cfg["window_size"])
+    gate = torch.sigmoid(xf @ params["gate.0.weight"].float().t())
+    o = gate[:, 0:1, None] * o_cmp + gate[:, 1:2, None] * o_sel + gate[:, 2:3, None] * o_win
+    y = o.reshape(o.shape[0], -1) @ params["proj_o.weight"].float().t()
+    return y, topk_idx, {"cmp": o_cmp, "sel": o_sel, "win": o_win, "gate": gate}
