@@ -24,6 +24,18 @@ sys.path.insert(0, os.path.join(ROOT, "flash-sparse-attention_amd"))
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 
+# HBM bytes per launch at the default workload from two rocprofv3 --pmc passes over this script
+# (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by the factor that makes the same counter
+# read 1 GiB for the 1 GiB device copy of --calib-copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
+PMC_TRAFFIC_BYTES = {
+    ("selattn_bwd_dqdkdv", 4): 14104562688,
+    ("selattn_fwd_main", 4): 8737412096,
+    ("selattn_fwd_main", 2): 4294666240,
+    ("selattn_fwd_main", 1): 2104956928,
+    ("selattn_fwd_reduce", 4): 5298789376,
+    ("selattn_bwd_dq_reduce", 4): 4575891456,
+}
+
 METRIC = "selected-attn fwd+bwd ms & TFLOP/s at 64K, B_K=64, T=16, GQA 1-4; roofline %"
 
 
@@ -36,6 +48,8 @@ def parse():
     ap.add_argument("--groups", type=str, default="1,2,4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seq-len", type=int, default=8192)
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="issue three 1 GiB device copies first (known-size reference for hardware counters)")
     return ap.parse_args()
 
 
@@ -102,6 +116,14 @@ def main():
     nblk = (n + bk - 1) // bk
     del own, lo, ok, nkeys
 
+    if args.calib_copy:
+        a = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        b = torch.empty_like(a)
+        for _ in range(3):
+            b.copy_(a)
+        torch.cuda.synchronize()
+        del a, b
+
     data = {}
     for g in groups:
         data[g] = tuple(x.to(dev) for x in make_qkv(n, hkv * g, hkv, d, dtype, seed=100 + g))
@@ -145,36 +167,50 @@ def main():
     kern = {k_: sum(v_) / len(v_) for k_, v_ in kern.items()}
 
     e = 2  # bytes per element
+    kv_once = 2 * n * hkv * d * e          # K and V (or dK and dV) of every kv head, once
+
     def algo(name, g):
+        """(flops, bytes) one launch must do at the least: MFMA flops over unmasked (query, key) pairs,
+        HBM bytes of the tensors it has to read and write once."""
         hq = hkv * g
-        fl = {"selattn_fwd_main": 4.0, "selattn_bwd_dq": 6.0, "selattn_bwd_dkdv": 4.0}
-        if name in fl:
-            return "mfma", fl[name] * d * p_key * g
+        pg = pairs * g                      # (query, head, block) rows
+        if name == "selattn_fwd_main":      # S = QK^T, O = PV; Q row in, normalised partial row + lse out
+            return 4.0 * d * p_key * g, pg * (2 * d * e + 4) + kv_once
+        if name == "selattn_bwd_dqdkdv":    # S, dP, dV, dK, dQ; Q, dO rows in, dQ partial row out, lse + delta in
+            return 10.0 * d * p_key * g, pg * (3 * d * e + 8) + 2 * kv_once
+        if name == "selattn_bwd_dq":
+            return 6.0 * d * p_key * g, pg * (3 * d * e + 8) + kv_once
+        if name == "selattn_bwd_dkdv":
+            return 8.0 * d * p_key * g, pg * (2 * d * e + 8) + 2 * kv_once
         if name == "selattn_fwd_reduce":
-            return "hbm", pairs * g * (d * e + 4) + n * hq * (d * e + 4)
+            return 0.0, pg * (d * e + 4) + n * hq * (d * e + 4)
         if name == "selattn_bwd_dq_reduce":
-            return "hbm", pairs * g * d * e + n * hq * d * e
+            return 0.0, pg * d * e + n * hq * d * e
         if name == "selattn_bwd_delta":
-            return "hbm", 2 * n * hq * d * e + n * hq * 4
+            return 0.0, 2 * n * hq * d * e + n * hq * 4
         if name == "index_build":
-            return "hbm", 4 * hkv * n * topk * 2 + 4 * (pairs + 2 * nblk * hkv)
+            return 0.0, 4 * hkv * n * topk * 2 + 4 * (pairs + 2 * nblk * hkv)
         if name == "selattn_bwd_dkdv_reduce":
-            return "hbm", 2 * n * hkv * d * e
-        return "hbm", 0.0
+            return 0.0, kv_once
+        return 0.0, 0.0
 
     kernels = []
     for (name, g), ms in sorted(kern.items(), key=lambda kv: -kv[1]):
-        bound, work = algo(name, g)
-        if bound == "mfma":
-            ach, peak, unit = work / (ms * 1e-3) / 1e12, MFMA_PEAK_TFLOPS, "TFLOP/s"
+        fl, by = algo(name, g)
+        tf, gbs = fl / (ms * 1e-3) / 1e12, by / (ms * 1e-3) / 1e9
+        f_mfma, f_hbm = tf / MFMA_PEAK_TFLOPS, gbs / HBM_PEAK_GBS
+        rec = {"kernel": name, "gqa": g, "ms": round(ms, 4)}
+        if f_mfma > f_hbm:                  # the roofline that binds is the one the kernel sits closer to
+            rec.update(bound="mfma", achieved=round(tf, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s", frac=round(f_mfma, 4))
         else:
-            ach, peak, unit = work / (ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"
-        kernels.append({"kernel": name, "gqa": g, "ms": round(ms, 4), "bound": bound,
-                        "achieved": round(ach, 2), "peak": peak, "unit": unit, "frac": round(ach / peak, 4)})
+            rec.update(bound="hbm", achieved=round(gbs, 2), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(f_hbm, 4))
+        rec.update(algo_tflops=round(tf, 2), algo_gbs=round(gbs, 1), algo_bytes=int(by))
+        kernels.append(rec)
     dom = kernels[0]
+    traffic = PMC_TRAFFIC_BYTES.get((dom["kernel"], dom["gqa"])) if (n, d, bk, topk) == (65536, 128, 64, 16) else None
     roofline = {"kernel": f"{dom['kernel']} (GQA {dom['gqa']})", "bound": dom["bound"],
                 "achieved": dom["achieved"], "peak": dom["peak"], "unit": dom["unit"], "frac": dom["frac"],
-                "traffic": None}
+                "traffic": traffic}
 
     per_gqa = []
     for g in groups:
