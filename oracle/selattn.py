@@ -13,6 +13,8 @@ Pinning status (tests/test_oracle_selattn.py):
   selected_attention_grads_ref : pinned - explicit backward formulas checked
       against autograd of the dense fp64 formulation, autograd of
       selected_attention_ref and central finite differences on tiny inputs.
+  selected_attention_rows_ref : pinned - equals the two functions above on
+      every row / block of small inputs (independent code path).
   build_index_ref : pinned - brute-force Python loops, torch.bincount,
       exclusive cumsum identity.
 """
@@ -184,6 +186,67 @@ def selected_attention_grads_ref(q, k, v, topk_idx, block_size, cu_seqlens, do, 
         dk[s0:s1] = dkb.reshape(Hkv, nblk * B, D)[:, :L].permute(1, 0, 2)
         dv[s0:s1] = dvb.reshape(Hkv, nblk * B, D)[:, :L].permute(1, 0, 2)
     return o_out, lse_out, dq, dk, dv
+
+
+def selected_attention_rows_ref(q, k, v, topk_idx, block_size, cu_seqlens, rows, do=None, softmax_scale=None,
+                                o_in=None, lse_in=None, round_dtype=None, key_block=None, dtype=torch.float64):
+    """The same quantities for a SAMPLE of queries, one explicit key list per (row, kv head).
+
+    rows: global query rows.  Returns dict with o [R,Hq,D], lse [Hq,R] (base 2) and, if `do` is given, dq [R,Hq,D]
+    plus - when key_block = (kv head, global first row of the block) - the sum over the sampled rows and the group's
+    heads of their contributions to dK and dV of that block's keys (dk_block, dv_block [B_K, D], rows beyond the
+    sequence end zero).  Written independently of the chunked functions above (no block views, no batched gathers)
+    so that either can check the other; same formulas and rounding points (see selected_attention_grads_ref)."""
+    def rnd(x):
+        return x if round_dtype is None else x.to(round_dtype).to(dtype)
+
+    N, Hq, D = q.shape
+    Hkv = k.shape[1]
+    g = Hq // Hkv
+    B = block_size
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    c = softmax_scale * LOG2E
+    bounds = _seq_bounds(cu_seqlens)
+    starts = np.array([b[0] for b in bounds])
+    R = len(rows)
+    out = {"o": torch.zeros(R, Hq, D, dtype=dtype), "lse": torch.full((Hq, R), float("-inf"), dtype=dtype)}
+    if do is not None:
+        out["dq"] = torch.zeros(R, Hq, D, dtype=dtype)
+        if key_block is not None:
+            out["dk_block"] = torch.zeros(B, D, dtype=dtype)
+            out["dv_block"] = torch.zeros(B, D, dtype=dtype)
+    for r, row in enumerate(int(x) for x in rows):
+        si = int(np.searchsorted(starts, row, side="right")) - 1
+        s0, s1 = bounds[si]
+        i, L = row - s0, s1 - s0
+        for kh in range(Hkv):
+            blocks = sorted({int(x) for x in topk_idx[kh, row] if int(x) >= 0 and int(x) * B <= i})
+            if not blocks:
+                continue
+            keys = torch.cat([torch.arange(x * B, min((x + 1) * B, i + 1, L)) for x in blocks]) + s0
+            kk, vv = k[keys, kh].to(dtype), v[keys, kh].to(dtype)
+            hs = slice(kh * g, (kh + 1) * g)
+            sc = (q[row, hs].to(dtype) @ kk.t()) * c                      # [g, nkeys]
+            lse = torch.logsumexp(sc / LOG2E, -1) * LOG2E
+            o = torch.exp2(sc - lse[:, None]) @ vv
+            out["o"][r, hs], out["lse"][hs, r] = o, lse
+            if do is None:
+                continue
+            lse_use = lse if lse_in is None else lse_in[hs, row].to(dtype)
+            o_use = o if o_in is None else o_in[row, hs].to(dtype)
+            dor = do[row, hs].to(dtype)
+            p = torch.exp2(sc - lse_use[:, None])
+            ds = softmax_scale * p * (dor @ vv.t() - (o_use * dor).sum(-1, keepdim=True))
+            ds_c, p_c = rnd(ds), rnd(p)
+            out["dq"][r, hs] = ds_c @ kk
+            if key_block is not None and key_block[0] == kh:
+                inblk = (keys >= key_block[1]) & (keys < key_block[1] + B)
+                if bool(inblk.any()):
+                    off = keys[inblk] - key_block[1]
+                    out["dk_block"][off] += ds_c[:, inblk].t() @ q[row, hs].to(dtype)
+                    out["dv_block"][off] += p_c[:, inblk].t() @ dor
+    return out
 
 
 def dense_mask(topk_idx: torch.Tensor, block_size: int, cu_seqlens) -> torch.Tensor:

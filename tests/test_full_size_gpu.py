@@ -1,0 +1,103 @@
+"""GPU parity at the full benchmark sizes, where the whole-tensor oracle would take minutes:
+
+* index lists bit-exact against the CPU oracle (a sort of N*T keys, cheap at any size);
+* O / LSE / dQ of a seeded SAMPLE of queries, and dK / dV of sampled key blocks, against the per-row oracle
+  (same tolerances as the small cases: 2e-2 bf16, 5e-3 fp16, LSE 1e-3, plus one output ulp for gradients);
+* size-independent identities over the WHOLE output:
+    - scaling V by 2 scales O by exactly 2 and leaves LSE bit-identical (powers of two commute with rounding
+      outside the subnormal range; bit-exact for bf16, one ulp for fp16);
+    - sum_p dV[p, kh] = sum over the group's heads and all queries of dO   (rows of P sum to one);
+    - sum <k, dK> = sum <q, dQ> per kv head   (both equal sum dS_ip s_ip / c: scale invariance of q.k).
+  A dropped tile, a wrong block or a double-counted row breaks one of them.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from fsa_hip import ops
+from fsa_hip.synth import make_qkv, make_topk_idx
+from oracle import selattn as orc
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
+ULP = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}
+
+CASES = [
+    # name, S, Hq, Hkv, D, B_K, T, dtype, std
+    ("C1-gqa4", 65536, 16, 4, 128, 64, 16, torch.bfloat16, 1.0),
+    ("C1-gqa1", 65536, 4, 4, 128, 64, 16, torch.bfloat16, 1.0),
+    ("C3", 131072, 4, 2, 256, 128, 8, torch.float16, 0.5),
+]
+
+
+@pytest.mark.parametrize("name,n,hq,hkv,d,bk,t,dtype,std", CASES)
+def test_selected_attention_full_size(dev, name, n, hq, hkv, d, bk, t, dtype, std):
+    print(f"case {name} S={n} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    g = hq // hkv
+    cu = [0, n]
+    q, k, v, do = make_qkv(n, hq, hkv, d, dtype, seed=11, std=std)
+    topk = make_topk_idx(cu, hkv, bk, t, seed=12)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    index = ops.build_index(topk.to(dev), cu_t, bk)
+    qd, kd, vd, dod = (x.to(dev) for x in (q, k, v, do))
+    o, lse = ops.selattn_fwd(qd, kd, vd, index)
+    dq, dk, dv = ops.selattn_bwd(qd, kd, vd, o, dod, lse, index)
+    o2, lse2 = ops.selattn_fwd(qd, kd, vd * 2, index)
+    torch.cuda.synchronize()
+
+    # index: bit-exact
+    cu_blocks, counts, starts, sel_tokens, slot_of = orc.build_index_ref(topk, cu, bk)
+    nb = int(cu_blocks[-1])
+    assert np.array_equal(index.cu_blocks.cpu().numpy(), cu_blocks)
+    assert np.array_equal(index.counts.cpu().numpy()[:, :nb], counts)
+    assert np.array_equal(index.starts.cpu().numpy()[:, : nb + 1], starts)
+    assert np.array_equal(index.sel_tokens.cpu().numpy(), sel_tokens)
+    assert np.array_equal(index.slot_of.cpu().numpy(), slot_of)
+
+    # whole-output identities
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert torch.equal(lse2, lse)
+    if dtype == torch.bfloat16:
+        assert torch.equal(o2, o * 2)
+    else:   # fp16 partial rows can be subnormal, where doubling no longer commutes with rounding: allow one ulp
+        assert ((o2.float() - 2 * o.float()).abs() <= 2.0 ** -10 * o2.float().abs() + 2.0 ** -20).all()
+    dof, dvf = dod.double(), dv.double()
+    lhs = dvf.sum(0)                                               # [Hkv, D]
+    rhs = dof.view(n, hkv, g, d).sum((0, 2))
+    half_ulp = ULP[dtype] / 2
+    walk = 6 * half_ulp * dvf.pow(2).sum(0).sqrt() + 1e-6          # random-walk bound of the output rounding
+    print(f"  sum dV identity: max dev {(lhs - rhs).abs().max().item():.3e}, bound min {walk.min().item():.3e}", flush=True)
+    assert ((lhs - rhs).abs() <= walk).all()
+    kdk = (kd.double() * dk.double()).sum((0, 2))                  # [Hkv]
+    qdq = (qd.double() * dq.double()).view(n, hkv, g, d).sum((0, 2, 3))
+    scale_ = (kd.double() * dk.double()).abs().sum((0, 2))
+    print(f"  <k,dK> vs <q,dQ>: {kdk.tolist()} vs {qdq.tolist()}", flush=True)
+    assert ((kdk - qdq).abs() <= 4 * half_ulp * scale_ / math.sqrt(n) * 8 + 1e-3).all()
+
+    # sampled queries
+    gen = torch.Generator().manual_seed(13)
+    rows = sorted(set([0, 1, bk - 1, bk, n - 1, n - bk] + torch.randint(0, n, (90,), generator=gen).tolist()))
+    oc, lc = o.float().cpu(), lse.cpu()
+    r = orc.selected_attention_rows_ref(q, k, v, topk, bk, cu, rows, do=do, o_in=oc, lse_in=lc, round_dtype=dtype)
+    eo = (oc[rows].double() - r["o"]).abs().max().item()
+    el = (lc[:, rows].double() - r["lse"]).abs().max().item()
+    dqg = dq.float().cpu()[rows].double()
+    edq = ((dqg - r["dq"]).abs() - ULP[dtype] * r["dq"].abs()).max().item()
+    print(f"  sampled rows: max|dO|={eo:.3e} max|dLSE|={el:.3e} dQ excess={edq:.3e}", flush=True)
+    assert eo <= TOL[dtype] and el <= 1e-3 and edq <= TOL[dtype]
+
+    # sampled key blocks (block 0 has every query: too many rows for the CPU; take moderately shared blocks)
+    nblk = (n + bk - 1) // bk
+    for kh, blk in [(0, nblk // 8), (hkv - 1, nblk // 2), (0, nblk - 1)]:
+        s0 = int(starts[kh, blk])
+        users = sel_tokens[kh][s0 : s0 + int(counts[kh, blk])].tolist()
+        rb = orc.selected_attention_rows_ref(q, k, v, topk, bk, cu, users, do=do, o_in=oc, lse_in=lc,
+                                             round_dtype=dtype, key_block=(kh, blk * bk))
+        for nm, got, want in (("dk", dk, rb["dk_block"]), ("dv", dv, rb["dv_block"])):
+            gb = got[blk * bk : (blk + 1) * bk, kh].float().cpu().double()
+            ex = ((gb - want).abs() - ULP[dtype] * want.abs()).max().item()
+            print(f"  block {blk} kv head {kh} ({len(users)} queries): {nm} max err {(gb - want).abs().max().item():.3e}", flush=True)
+            assert ex <= TOL[dtype], (nm, blk, ex)

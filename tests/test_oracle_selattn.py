@@ -198,3 +198,22 @@ def test_synthetic_index_matches_stated_counts():
     assert (valid.sum(-1) == torch.minimum(own + 1, torch.tensor(16))[None]).all()
     srt = torch.where(valid, topk, torch.full_like(topk, 10**6)).sort(-1).values
     assert (torch.where(valid, topk, torch.full_like(topk, 10**6)) == srt).all()
+
+
+def test_rows_ref_equals_chunked_oracle():
+    """The per-row sampler (explicit key lists) and the chunked oracle (block views, batched gathers) agree on every
+    row and on the dK/dV of every block of a small ragged batch."""
+    from fsa_hip.synth import make_qkv, make_topk_idx
+    cu = [0, 150, 150, 391]
+    n, hq, hkv, d, bk, t = cu[-1], 4, 2, 32, 16, 4
+    q, k, v, do = make_qkv(n, hq, hkv, d, torch.float32, seed=5)
+    idx = make_topk_idx(cu, hkv, bk, t, seed=6)
+    o, lse, dq, dk, dv = orc.selected_attention_grads_ref(q, k, v, idx, bk, cu, do, dtype=torch.float64)
+    rows = list(range(n))
+    for kh, first in [(0, 0), (1, 150 + 3 * bk), (1, 150 + 15 * bk), (0, 9 * bk)]:
+        r = orc.selected_attention_rows_ref(q, k, v, idx, bk, cu, rows, do=do, key_block=(kh, first))
+        assert torch.allclose(r["o"], o, atol=1e-10) and torch.allclose(r["lse"], lse, atol=1e-10)
+        assert torch.allclose(r["dq"], dq, atol=1e-10)
+        hi = min(first + bk, 150 if first < 150 else n)
+        assert torch.allclose(r["dk_block"][: hi - first], dk[first:hi, kh], atol=1e-9)
+        assert torch.allclose(r["dv_block"][: hi - first], dv[first:hi, kh], atol=1e-9)
