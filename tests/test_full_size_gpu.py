@@ -101,3 +101,78 @@ def test_selected_attention_full_size(dev, name, n, hq, hkv, d, bk, t, dtype, st
             ex = ((gb - want).abs() - ULP[dtype] * want.abs()).max().item()
             print(f"  block {blk} kv head {kh} ({len(users)} queries): {nm} max err {(gb - want).abs().max().item():.3e}", flush=True)
             assert ex <= TOL[dtype], (nm, blk, ex)
+
+
+def test_decode_full_size(dev):
+    """One decode step at the full serving shape: 64 requests, cache lengths uniform in [32768, 131072], Hq=32,
+    Hkv=8, D=128, compression 32/16, B_K=64, T=16, bf16.  Caches are drawn on the device (21 GB); the oracle is run
+    on sampled requests (shortest, longest, first, last) from their slices, the top-k rule on every request, and
+    the batch is checked for independence of its requests (a sub-batch gives bit-identical results)."""
+    from oracle import decode as dorc
+    hq, hkv, d, bk, t, ks, st = 32, 8, 128, 64, 16, 32, 16
+    nreq = 64
+    gen = torch.Generator().manual_seed(31)
+    lens = torch.randint(32768, 131073, (nreq,), generator=gen).tolist()
+    cu_k, cu_ck = [0], [0]
+    for l in lens:
+        cu_k.append(cu_k[-1] + l)
+        cu_ck.append(cu_ck[-1] + (l - ks) // st + 1)
+    print(f"case decode B={nreq} total cache rows {cu_k[-1]} compressed rows {cu_ck[-1]}", flush=True)
+    torch.manual_seed(32)
+    q = torch.randn(nreq, hq, d, device=dev, dtype=torch.bfloat16)
+    kc = torch.randn(cu_k[-1], hkv, d, device=dev, dtype=torch.bfloat16)
+    vc = torch.randn(cu_k[-1], hkv, d, device=dev, dtype=torch.bfloat16)
+    ck = torch.randn(cu_ck[-1], hkv, d, device=dev, dtype=torch.bfloat16)
+    cv = torch.randn(cu_ck[-1], hkv, d, device=dev, dtype=torch.bfloat16)
+    pos = torch.tensor([l - 1 for l in lens], dtype=torch.int32, device=dev)
+    seqlens = torch.tensor(lens, dtype=torch.int32, device=dev)
+    cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)
+    cu_ck_t = torch.tensor(cu_ck, dtype=torch.int32, device=dev)
+    max_ck = max(b_ - a_ for a_, b_ in zip(cu_ck[:-1], cu_ck[1:]))
+    nblk_max = max(math.ceil(l / bk) for l in lens)
+
+    def step(sl):
+        b0, b1 = sl.start, sl.stop
+        cck = (cu_ck_t[b0 : b1 + 1] - cu_ck_t[b0]).contiguous()
+        ckk = (cu_k_t[b0 : b1 + 1] - cu_k_t[b0]).contiguous()
+        o_c, lse_c, raw = ops.decode_cmpattn(q[sl], ck[cu_ck[b0]:cu_ck[b1]], cv[cu_ck[b0]:cu_ck[b1]], cck, pos[sl],
+                                             ks, st, max_ck)
+        idx, bscore = ops.decode_topk(raw, lse_c, cck, pos[sl], seqlens[sl], hq, ks, st, bk, t, nblk_max,
+                                      softmax_scale=1.0 / math.sqrt(d), return_block_score=True)
+        o_s, lse_s = ops.decode_selattn(q[sl], kc[cu_k[b0]:cu_k[b1]], vc[cu_k[b0]:cu_k[b1]], ckk, idx, bk)
+        return o_c, lse_c, idx, bscore, o_s, lse_s
+
+    full = step(slice(0, nreq))
+    part = step(slice(5, 13))
+    torch.cuda.synchronize()
+    for a, b in zip(full, part):
+        a = a[5:13] if a.shape[0] == nreq else a[:, 5:13]
+        assert torch.equal(a, b)
+    o_c, lse_c, idx, bscore, o_s, lse_s = full
+    assert torch.isfinite(o_c.float()).all() and torch.isfinite(o_s.float()).all()
+    assert torch.equal(idx.cpu(), dorc.decode_topk_ref(bscore.cpu(), t))
+    # every request keeps block 0 and its last two blocks (init_blocks = 1, local_blocks = 2)
+    own = (seqlens.long() - 1) // bk
+    for forced in (torch.zeros_like(own), own, own - 1):
+        assert (idx.long() == forced[None, :, None]).any(-1).all()
+    order = sorted(range(nreq), key=lambda i: lens[i])
+    for b in sorted({order[0], order[-1], 0, nreq - 1}):
+        qb = q[b : b + 1].float().cpu()
+        ckb, cvb = (x[cu_ck[b]:cu_ck[b + 1]].float().cpu() for x in (ck, cv))
+        n_ck = cu_ck[b + 1] - cu_ck[b]
+        o_r, lse_r = dorc.decode_compressed_attention_ref(qb, ckb, cvb, [0, n_ck], [lens[b] - 1], ks, st)
+        e1 = (o_c[b : b + 1].float().cpu() - o_r).abs().max().item()
+        e2 = (lse_c[:, b : b + 1].cpu() - lse_r).abs().max().item()
+        bs_r = dorc.decode_block_scores_ref(qb, ckb, lse_r, [0, n_ck], [lens[b] - 1], [lens[b]], ks, st, bk,
+                                            nblk_cols=nblk_max)
+        got = bscore[:, b : b + 1].cpu()
+        assert torch.equal(torch.isinf(got), torch.isinf(bs_r))
+        fin = torch.isfinite(bs_r)
+        e3 = (got[fin] - bs_r[fin]).abs().max().item()
+        kcb, vcb = (x[cu_k[b]:cu_k[b + 1]].cpu() for x in (kc, vc))
+        o_sr, lse_sr = dorc.decode_selected_attention_ref(qb, kcb, vcb, [0, lens[b]], idx[:, b : b + 1].cpu(), bk)
+        e4 = (o_s[b : b + 1].float().cpu() - o_sr).abs().max().item()
+        e5 = (lse_s[:, b : b + 1].cpu() - lse_sr).abs().max().item()
+        print(f"  request {b} (len {lens[b]}): cmp dO {e1:.2e} dLSE {e2:.2e} block-score {e3:.2e}; "
+              f"sel dO {e4:.2e} dLSE {e5:.2e}", flush=True)
+        assert e1 <= 2e-2 and e2 <= 1e-3 and e3 <= 2e-3 and e4 <= 2e-2 and e5 <= 1e-3
