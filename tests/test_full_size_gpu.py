@@ -176,3 +176,45 @@ def test_decode_full_size(dev):
         print(f"  request {b} (len {lens[b]}): cmp dO {e1:.2e} dLSE {e2:.2e} block-score {e3:.2e}; "
               f"sel dO {e4:.2e} dLSE {e5:.2e}", flush=True)
         assert e1 <= 2e-2 and e2 <= 1e-3 and e3 <= 2e-3 and e4 <= 2e-2 and e5 <= 1e-3
+
+
+def test_module_full_size(dev):
+    """The Llama-3-8B-like layer at its full shape (hidden 4096, 32 / 8 heads of 128, compression 32/16, B_K=64,
+    T=16, window 512; 4 sequences of 8192 tokens, bf16), forward and backward.  Every branch is causal, so the
+    output of the first 1024 tokens of a sequence depends on those tokens only: that prefix is checked against the
+    CPU oracle of the layer, for the first and the last sequence; the varlen batch is checked against a run of one
+    of its sequences alone."""
+    from fsa.module.fsa import FlashSparseAttention, RopeConfig
+    from oracle import module as morc
+    torch.manual_seed(3)
+    cfg = dict(hidden_size=4096, num_q_heads=32, num_kv_heads=8, head_dim=128, kernel_size=32, kernel_stride=16,
+               block_size=64, topk=16, init_blocks=1, local_blocks=2, window_size=512)
+    layer = FlashSparseAttention(**cfg, rope_config=RopeConfig(head_dim=128)).to(dev).to(torch.bfloat16)
+    nseq, slen, pre = 4, 8192, 1024
+    n = nseq * slen
+    x = torch.randn(n, 4096, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    cu = torch.arange(0, n + 1, slen, dtype=torch.int32, device=dev)
+    print(f"case module {nseq} x {slen}", flush=True)
+    y, topk_idx = layer(x, cu, return_topk_idx=True)
+    (y.float() * torch.randn_like(y, dtype=torch.float32)).sum(-1).mean().backward()
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all() and torch.isfinite(x.grad.float()).all()
+    for name, p in layer.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad.float()).all() and p.grad.abs().max() > 0, name
+
+    def rel(a, b):
+        return ((a.float() - b.float()).norm() / b.float().norm()).item()
+
+    with torch.no_grad():
+        y1 = layer(x[2 * slen : 3 * slen].detach(), cu[:2])
+    e = rel(y[2 * slen : 3 * slen], y1)
+    print(f"  sequence 2 alone vs in the batch: rel {e:.3e}", flush=True)
+    assert e < 1e-2
+    params = {k: v.detach().float().cpu() for k, v in layer.named_parameters()}
+    ocfg = dict(cfg, inv_freq=morc.llama3_inv_freq(128, 500000.0))
+    for s in (0, nseq - 1):
+        xs = x[s * slen : s * slen + pre].detach().float().cpu()
+        y_r, _, _ = morc.fsa_layer_ref(params, xs, [0, pre], ocfg, topk_idx=topk_idx[:, s * slen : s * slen + pre].cpu())
+        e = rel(y[s * slen : s * slen + pre].cpu(), y_r)
+        print(f"  sequence {s} first {pre} tokens vs oracle: rel {e:.3e}", flush=True)
+        assert e < 2e-2
