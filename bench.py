@@ -48,6 +48,9 @@ def parse():
     ap.add_argument("--groups", type=str, default="1,2,4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seq-len", type=int, default=8192)
+    ap.add_argument("--workload", choices=["c1", "c3", "module", "decode"], default="c1",
+                    help="c1 = the headline configuration (default); the others time the remaining parity "
+                         "configurations (large-head fp16 selected attention, the full layer, one decode step)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="issue three 1 GiB device copies first (known-size reference for hardware counters)")
     return ap.parse_args()
@@ -84,12 +87,86 @@ def cpu_baseline(seq_len: int, d: int, bk: int, topk: int, hkv: int):
     }
 
 
+def side_workload(args):
+    """Timing of the two parity configurations that are not selected attention alone: the full layer
+    (forward + backward, 4 x 8192 tokens) and one decode step (64 requests).  Same JSON shape, value in ms."""
+    import math
+    import torch
+    from fsa_hip import _lib, ops
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    if args.workload == "module":
+        from fsa.module.fsa import FlashSparseAttention, RopeConfig
+        layer = FlashSparseAttention(hidden_size=4096, num_q_heads=32, num_kv_heads=8, head_dim=128, kernel_size=32,
+                                     kernel_stride=16, block_size=64, topk=16, init_blocks=1, local_blocks=2,
+                                     window_size=512, rope_config=RopeConfig(head_dim=128)).to(dev).to(torch.bfloat16)
+        n = 4 * 8192
+        x = torch.randn(n, 4096, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        w = torch.randn(n, 4096, device=dev, dtype=torch.bfloat16)
+        cu = torch.arange(0, n + 1, 8192, dtype=torch.int32, device=dev)
+        name = "FlashSparseAttention layer fwd+bwd, hidden 4096, Hq=32, Hkv=8, D=128, 32/16 compression, B_K=64, " \
+               "T=16, window 512, 4 x 8192 tokens"
+
+        def step():
+            layer.zero_grad(set_to_none=True)
+            x.grad = None
+            (layer(x, cu) * w).sum().backward()
+    else:
+        hq, hkv, d, bk, t, ks, st, nreq = 32, 8, 128, 64, 16, 32, 16, 64
+        gen = torch.Generator().manual_seed(31)
+        lens = torch.randint(32768, 131073, (nreq,), generator=gen).tolist()
+        cu_k, cu_ck = [0], [0]
+        for l in lens:
+            cu_k.append(cu_k[-1] + l)
+            cu_ck.append(cu_ck[-1] + (l - ks) // st + 1)
+        q = torch.randn(nreq, hq, d, device=dev, dtype=torch.bfloat16)
+        kc, vc = (torch.randn(cu_k[-1], hkv, d, device=dev, dtype=torch.bfloat16) for _ in range(2))
+        ck, cv = (torch.randn(cu_ck[-1], hkv, d, device=dev, dtype=torch.bfloat16) for _ in range(2))
+        pos = torch.tensor([l - 1 for l in lens], dtype=torch.int32, device=dev)
+        seqlens = torch.tensor(lens, dtype=torch.int32, device=dev)
+        cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)
+        cu_ck_t = torch.tensor(cu_ck, dtype=torch.int32, device=dev)
+        max_ck = max(b - a for a, b in zip(cu_ck[:-1], cu_ck[1:]))
+        nblk_max = max(math.ceil(l / bk) for l in lens)
+        name = f"one decode step (compressed attention, top-k, selected attention), {nreq} requests, caches " \
+               f"32768-131072 ({cu_k[-1]} rows), Hq=32, Hkv=8, D=128, B_K=64, T=16"
+
+        def step():
+            o_c, lse_c, raw = ops.decode_cmpattn(q, ck, cv, cu_ck_t, pos, ks, st, max_ck)
+            idx = ops.decode_topk(raw, lse_c, cu_ck_t, pos, seqlens, hq, ks, st, bk, t, nblk_max,
+                                  softmax_scale=1.0 / math.sqrt(d))
+            ops.decode_selattn(q, kc, vc, cu_k_t, idx, bk)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    _lib.profile_enable(True)
+    step()
+    torch.cuda.synchronize()
+    recs = _lib.profile_records()
+    _lib.profile_enable(False)
+    kern = {}
+    for nm, t_ in recs:
+        kern[nm] = kern.get(nm, 0.0) + t_
+    print(json.dumps({"metric": "ms per step", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": name},
+                      "library_kernels_ms": {k_: round(v_, 4) for k_, v_ in sorted(kern.items(), key=lambda kv: -kv[1])}}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (every box has one GPU); run with --gpus 1",
               file=sys.stderr)
         sys.exit(2)
+    if args.workload in ("module", "decode"):
+        return side_workload(args)
     import torch
     from fsa.ops.FSA_topk_sparse_attention import (_topk_sparse_attention_bwd_opt,
                                                    _topk_sparse_attention_fwd_opt)
@@ -100,7 +177,9 @@ def main():
     dev = torch.device("cuda:0")
     n, hkv, d, bk, topk = args.seq_len, 4, 128, 64, 16
     groups = [int(x) for x in args.groups.split(",")]
-    dtype = torch.bfloat16
+    dtype, std = torch.bfloat16, 1.0
+    if args.workload == "c3":           # large heads: fp16, D=256, Hkv=2, GQA 2, S=131072, B_K=128, T=8, sigma 0.5
+        n, hkv, d, bk, topk, groups, dtype, std = 131072, 2, 256, 128, 8, [2], torch.float16, 0.5
     scale = 1.0 / d ** 0.5
     cu = [0, n]
     cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
@@ -126,7 +205,7 @@ def main():
 
     data = {}
     for g in groups:
-        data[g] = tuple(x.to(dev) for x in make_qkv(n, hkv * g, hkv, d, dtype, seed=100 + g))
+        data[g] = tuple(x.to(dev) for x in make_qkv(n, hkv * g, hkv, d, dtype, seed=100 + g, std=std))
 
     def run_g(g):
         q, k, v, do = data[g]
@@ -234,7 +313,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "bf16" if dtype == torch.bfloat16 else "fp16",
         "data": "synthetic",
         "config": {"workload": f"selected attention index+fwd+bwd, 1 varlen sequence S={n}, Hkv={hkv}, "
                                f"GQA {'/'.join(map(str, groups))} swept in one step, D={d}, B_K={bk}, T={topk}",
@@ -245,7 +324,7 @@ def main():
         "per_gqa": per_gqa,
         "kernels": kernels,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.workload == "c1":
         out["cpu_baseline"] = cpu_baseline(args.cpu_seq_len, d, bk, topk, hkv)
     print(json.dumps(out))
 

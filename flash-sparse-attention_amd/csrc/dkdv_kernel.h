@@ -89,12 +89,13 @@ template <int MODE, int BK> struct KvBlock {
 };
 
 // ----------------------------------------------------------------- dkdv ----
-constexpr int KV_R = 64;             // gathered rows per pass
 constexpr int KV_TILE_ROWS = 4096;   // rows per work-group and head of the group (scaled by g, capped)
 static inline int kv_tile_rows(int g) { return KV_TILE_ROWS * (g < 2 ? g : 2); }
 
 template <int D, int BK> struct KvCfg {
   static constexpr int NW = BK / 16;        // one wave per 16 keys
+  // gathered rows per pass; 32 where 8 waves of head_dim 256 leave no registers for a 64-row pass
+  static constexpr int KV_R = (D >= 256 && BK >= 128) ? 32 : 64;
   static constexpr int NT = NW * 64;
   static constexpr int QS = D + 8;         // LDS row stride of the Q / dO tiles (16 B pad; a larger pad would push two work-groups past 160 KB of LDS)
   static constexpr int CPR = D / 8;         // 16-byte chunks per row
@@ -104,9 +105,20 @@ template <int D, int BK> struct KvCfg {
   // with the fused dQ: K of the block (natural layout) and the dS^T tile [BK][KV_R]
   static constexpr int KS = D + 8;
   static constexpr int DSS = KV_R + 8;
-  static constexpr bool STAGE_DQ = BYTES + (BK * KS + BK * DSS + NW * 16 * QS) * 2 <= 160 * 1024;
-  static constexpr int BYTES_FUSED = BYTES + (BK * KS + BK * DSS + (STAGE_DQ ? NW * 16 * QS : 0)) * 2;  // + per-wave dQ staging tiles
+  // fused dQ: row tiles (16 rows) are dealt to the waves; with more waves than row tiles, TG waves share a
+  // row tile and split its d tiles.  Each wave stages its [16][DW] piece for row-coalesced stores.
+  static constexpr int NRT = KV_R / 16;
+  static constexpr int TG = NW > NRT ? NW / NRT : 1;
+  static constexpr int RW = NW / TG;                 // waves that start on distinct row tiles
+  static constexpr int DW = D / TG;                  // columns of dQ per wave
+  static constexpr int DQS = DW + 8;
+  static constexpr bool STAGE_DQ = BYTES + (BK * KS + BK * DSS + NW * 16 * DQS) * 2 <= 160 * 1024;
+  static constexpr int BYTES_FUSED = BYTES + (BK * KS + BK * DSS + (STAGE_DQ ? NW * 16 * DQS : 0)) * 2;
   static constexpr int MIN_WAVES = (D <= 128 && NT <= 256) ? 2 : 1;  // work-groups per CU the registers allow
+  // with 8 waves the register budget is 256 per lane: K fragments are then re-read from the LDS copy of the
+  // block that the fused dQ keeps anyway, instead of living in 32 registers
+  static constexpr bool K_FROM_LDS = D >= 256 && NT >= 512;
+  static constexpr bool TIGHT_REGS = D >= 256 && NT >= 512;
   static_assert(KV_R * CPR % NT == 0, "tile must divide evenly over the threads");
 };
 
@@ -114,22 +126,26 @@ template <int D, int BK> struct KvCfg {
 // its (query, block) pairs - dQ^T = K^T dS^T with dS^T exchanged between the
 // waves through LDS - so Q and dO are gathered once for dQ, dK and dV.
 template <typename T, int D, int BK, int MODE, bool FUSE_DQ = false>
+#ifndef KV_LB_PROBE
 __global__ void __launch_bounds__((KvCfg<D, BK>::NT), (KvCfg<D, BK>::MIN_WAVES))
+#else
+__global__ void __launch_bounds__(256)
+#endif
 attn_bwd_dkdv_kernel(SelBwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
   typedef KvCfg<D, BK> C;
-  constexpr int QS = C::QS, NS = D / 32, NDT = D / 16, NRT = KV_R / 16, NU = KV_R / 32;
+  constexpr int QS = C::QS, NS = D / 32, NDT = D / 16, NRT = C::NRT, NU = C::KV_R / 32;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* Qs = reinterpret_cast<T*>(smem);
-  T* Os = Qs + KV_R * QS;
-  float* lse_s = reinterpret_cast<float*>(Os + KV_R * QS);
-  float* del_s = lse_s + KV_R;
-  int* lim_s = reinterpret_cast<int*>(del_s + KV_R);
-  int* llo_s = lim_s + KV_R;
-  T* Kl = reinterpret_cast<T*>(llo_s + KV_R);   // FUSE_DQ only
+  T* Os = Qs + C::KV_R * QS;
+  float* lse_s = reinterpret_cast<float*>(Os + C::KV_R * QS);
+  float* del_s = lse_s + C::KV_R;
+  int* lim_s = reinterpret_cast<int*>(del_s + C::KV_R);
+  int* llo_s = lim_s + C::KV_R;
+  T* Kl = reinterpret_cast<T*>(llo_s + C::KV_R);   // FUSE_DQ only
   T* dSs = Kl + BK * C::KS;                     // FUSE_DQ only
-  T* dQst = dSs + BK * C::DSS + (threadIdx.x >> 6) * (16 * C::QS);  // FUSE_DQ only: this wave's [16][D] tile
+  T* dQst = dSs + BK * C::DSS + (threadIdx.x >> 6) * (16 * C::DQS);  // FUSE_DQ only: this wave's [16][DW] tile
 
   const int h = blockIdx.y;
   const int64_t nbp1 = p.max_blocks + 1;
@@ -152,16 +168,17 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   const bool key_ok = key < blk.n_keys_valid;
 
   // K / V fragments of this wave's 16 keys stay in registers: B[k = d][n = key]
-  vec8 kf[NS], vf[NS];
+  constexpr bool KLDS = FUSE_DQ && C::K_FROM_LDS;
+  vec8 kf[KLDS ? 1 : NS], vf[NS];
   {
     const T* krow = reinterpret_cast<const T*>(p.k) + (int64_t)ktok * p.k_sn + (int64_t)h * p.k_sh + 8 * kg;
     const T* vrow = reinterpret_cast<const T*>(p.v) + (int64_t)ktok * p.v_sn + (int64_t)h * p.v_sh + 8 * kg;
 #pragma unroll
     for (int s_ = 0; s_ < NS; ++s_) {
-      kf[s_] = zero8<T>();
+      if (!KLDS) kf[s_] = zero8<T>();
       vf[s_] = zero8<T>();
       if (key_ok) {
-        kf[s_] = load16<vec8>(krow + 32 * s_);
+        if (!KLDS) kf[s_] = load16<vec8>(krow + 32 * s_);
         vf[s_] = load16<vec8>(vrow + 32 * s_);
       }
     }
@@ -196,7 +213,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       const int r = base + ld_row + C::ROW_STEP * j;
       tok_pf[j] = r < row_hi ? row_token(r) : 0;
     }
-    if (tid < KV_R) tok_stat = base + tid < row_hi ? row_token(base + tid) : 0;
+    if (tid < C::KV_R) tok_stat = base + tid < row_hi ? row_token(base + tid) : 0;
   };
   // global -> registers for the pass starting at row `base` (its token ids are in tok_pf)
   auto fetch = [&](int base) {
@@ -212,7 +229,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         dost[j] = load16<vec8>(dobase + (int64_t)token * p.do_sn + (int64_t)head * p.do_sh + ld_col * 8);
       }
     }
-    if (tid < KV_R) {
+    if (tid < C::KV_R) {
       const int r = base + tid;
       lse_st = INFINITY;  // rows past the end: P = exp2(s - inf) = 0
       del_st = 0.f;
@@ -236,7 +253,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       store16(&Qs[row * QS + ld_col * 8], qst[j]);
       store16(&Os[row * QS + ld_col * 8], dost[j]);
     }
-    if (tid < KV_R) {
+    if (tid < C::KV_R) {
       lse_s[tid] = lse_st;
       del_s[tid] = del_st;
       lim_s[tid] = lim_st;
@@ -259,14 +276,14 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 
   fetch_tokens(row_lo);
   fetch(row_lo);
-  fetch_tokens(row_lo + KV_R);
+  fetch_tokens(row_lo + C::KV_R);
   stash();
   __syncthreads();
-  for (int base = row_lo; base < row_hi; base += KV_R) {
-    const bool more = base + KV_R < row_hi;
+  for (int base = row_lo; base < row_hi; base += C::KV_R) {
+    const bool more = base + C::KV_R < row_hi;
     if (more) {
-      fetch(base + KV_R);
-      fetch_tokens(base + 2 * KV_R);
+      fetch(base + C::KV_R);
+      fetch_tokens(base + 2 * C::KV_R);
     }
 
     vec4 pk[NRT], dsk[NRT];
@@ -276,9 +293,10 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 #pragma unroll
       for (int s_ = 0; s_ < NS; ++s_) {
         vec8 qa = load16<vec8>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
-        sacc = Elem<T>::mfma16(qa, kf[s_], sacc);
+        sacc = Elem<T>::mfma16(qa, KLDS ? load16<vec8>(&Kl[key * C::KS + 32 * s_ + 8 * kg]) : kf[KLDS ? 0 : s_], sacc);
         vec8 da = load16<vec8>(&Os[rt * 16 * QS + a_off + 32 * s_]);
         dpacc = Elem<T>::mfma16(da, vf[s_], dpacc);
+        if (C::TIGHT_REGS && (s_ & 1) == 1) asm volatile("" ::: "memory");
       }
       const float4 lse4 = *reinterpret_cast<const float4*>(&lse_s[rt * 16 + 4 * kg]);
       const float4 del4 = *reinterpret_cast<const float4*>(&del_s[rt * 16 + 4 * kg]);
@@ -316,6 +334,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
         vec8 qa = lds_read_tr8<T>(&Qs[32 * u * QS + tr_off + 16 * t], 16 * QS);
         dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
+        if (C::TIGHT_REGS && (t & 1) == 1) asm volatile("" ::: "memory");  // keep the operand reads from piling up
       }
     }
     if (FUSE_DQ) {
@@ -325,13 +344,16 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       const int64_t prow0 = ((int64_t)h * p.cap + start) * p.g;
       const int ktr_off = (4 * kg + (l16 >> 2)) * C::KS + 4 * (l16 & 3);   // + 32*u*KS + 16*t
       const int str_off = (4 * kg + (l16 >> 2)) * C::DSS + 4 * (l16 & 3);  // + 32*u*DSS + 16*rt
-      for (int rt = wv; rt < NRT; rt += C::NW) {
+      const int tg = wv / C::RW;                     // which share of the d tiles
+      constexpr int NTW = NDT / C::TG;               // d tiles per wave
+      for (int rt = wv % C::RW; rt < NRT; rt += C::RW) {
         vec8 dsb[BK / 32];
 #pragma unroll
         for (int u = 0; u < BK / 32; ++u)
           dsb[u] = lds_read_tr8<T>(&dSs[32 * u * C::DSS + str_off + 16 * rt], 16 * C::DSS);
 #pragma unroll
-        for (int t = 0; t < NDT; ++t) {
+        for (int tt = 0; tt < NTW; ++tt) {
+          const int t = tg * NTW + tt;
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int u = 0; u < BK / 32; ++u) {
@@ -342,21 +364,21 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) x[i] = (T)acc[i];
           if (C::STAGE_DQ) {
-            store8(&dQst[l16 * QS + 16 * t + 4 * kg], x);
+            store8(&dQst[l16 * C::DQS + 16 * tt + 4 * kg], x);
           } else {  // LDS too small for the staging tiles: direct 8-byte stores
             const int r = base + rt * 16 + l16;
             if (r < row_hi) store8(dqpart + (prow0 + r) * D + 16 * t + 4 * kg, x);
           }
         }
-        // [16 rows][D] tile -> row-coalesced 16-byte stores (CPR lanes per row)
+        // [16 rows][DW] piece -> row-coalesced 16-byte stores (CPW lanes per row)
         __builtin_amdgcn_wave_barrier();
-        constexpr int RPI = 64 / C::CPR;
+        constexpr int CPW = C::DW / 8, RPI = 64 / CPW;
 #pragma unroll
         for (int j = 0; C::STAGE_DQ && j < 16 / RPI; ++j) {
-          const int row = lane / C::CPR + RPI * j;
+          const int row = lane / CPW + RPI * j;
           const int r = base + rt * 16 + row;
-          vec8 x = load16<vec8>(&dQst[row * QS + (lane % C::CPR) * 8]);
-          if (r < row_hi) store16(dqpart + (prow0 + r) * D + (lane % C::CPR) * 8, x);
+          vec8 x = load16<vec8>(&dQst[row * C::DQS + (lane % CPW) * 8]);
+          if (r < row_hi) store16(dqpart + (prow0 + r) * D + tg * C::DW + (lane % CPW) * 8, x);
         }
         __builtin_amdgcn_wave_barrier();
       }

@@ -123,19 +123,20 @@ lc_fwd_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __re
     }
 }
 
-// bias[h, dout] = sum_{k,d} pe[h,k,d] W[h,k,d,dout]  (fp32 accumulation, rounded once)
+// bias[h, dout] = sum_{k,d} pe[h,k,d] W[h,k,d,dout]  (fp32 accumulation, rounded once).
+// One work-group per (head, 8 output columns): 32 row slices x 8 columns, slices summed in a fixed order.
 template <typename T>
 __global__ void __launch_bounds__(256)
 lc_bias_kernel(const T* __restrict__ pe, const T* __restrict__ w, T* __restrict__ bias, int kd, int d) {
   __shared__ float part[256];
   const int h = blockIdx.x, tid = threadIdx.x;
-  const int dout = tid % d, slice = tid / d, nslice = 256 / d;
+  const int c = tid & 7, slice = tid >> 3, dout = blockIdx.y * 8 + c;
   float s = 0.f;
-  for (int i = slice; i < kd; i += nslice) s += (float)pe[(int64_t)h * kd + i] * (float)w[((int64_t)h * kd + i) * d + dout];
+  for (int i = slice; i < kd; i += 32) s += (float)pe[(int64_t)h * kd + i] * (float)w[((int64_t)h * kd + i) * d + dout];
   part[tid] = s;
   __syncthreads();
   if (slice == 0) {
-    for (int j = 1; j < nslice; ++j) s += part[j * d + dout];
+    for (int j = 1; j < 32; ++j) s += part[j * 8 + c];
     bias[h * d + dout] = (T)s;
   }
 }
@@ -201,13 +202,13 @@ __global__ void __launch_bounds__(256)
 lc_dbias_kernel(const T* __restrict__ dy, float* __restrict__ dbias, int64_t ny_total, int nheads, int d) {
   __shared__ float part[256];
   const int h = blockIdx.x, tid = threadIdx.x;
-  const int dout = tid % d, slice = tid / d, nslice = 256 / d;
+  const int c = tid & 7, slice = tid >> 3, dout = blockIdx.y * 8 + c;
   float s = 0.f;
-  for (int64_t n = slice; n < ny_total; n += nslice) s += (float)dy[(n * nheads + h) * d + dout];
+  for (int64_t n = slice; n < ny_total; n += 32) s += (float)dy[(n * nheads + h) * d + dout];
   part[tid] = s;
   __syncthreads();
   if (slice == 0) {
-    for (int j = 1; j < nslice; ++j) s += part[j * d + dout];
+    for (int j = 1; j < 32; ++j) s += part[j * 8 + c];
     dbias[h * d + dout] = s;
   }
 }
@@ -328,7 +329,7 @@ static int lc_fwd_t(const void* x, int64_t x_sn, int64_t x_sh, const void* w, co
                     int ks, int stride, hipStream_t stream) {
   if (pe) {
     ProfScope ps_("linear_compress_bias", stream);
-    lc_bias_kernel<T><<<h, 256, 0, stream>>>((const T*)pe, (const T*)w, (T*)bias, ks * d, d);
+    lc_bias_kernel<T><<<dim3(h, d / 8), 256, 0, stream>>>((const T*)pe, (const T*)w, (T*)bias, ks * d, d);
   }
   dim3 grid((unsigned)((max_y + LC_ROWS - 1) / LC_ROWS), batch, h);
   ProfScope ps_("linear_compress_fwd", stream);
@@ -378,7 +379,7 @@ static int lc_bwd_t(const void* x, int64_t x_sn, int64_t x_sh, const void* w, co
   }
   if (pe) {
     ProfScope ps_("linear_compress_dbias", stream);
-    lc_dbias_kernel<T><<<h, 256, 0, stream>>>((const T*)dy, dbias, total_y, h, d);
+    lc_dbias_kernel<T><<<dim3(h, d / 8), 256, 0, stream>>>((const T*)dy, dbias, total_y, h, d);
     lc_dpe_kernel<T><<<dim3((ks * d + 255) / 256, h), 256, 0, stream>>>((const T*)w, dbias, (T*)dpe, ks * d, d);
   }
   {
