@@ -85,7 +85,7 @@ template <int MODE> struct KeyRange {
 
 // ---------------------------------------------------------------- forward ----
 template <typename T, int D, int MODE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1))
 cmpattn_fwd_kernel(CmpParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
@@ -200,7 +200,7 @@ cmpattn_fwd_kernel(CmpParams p) {
 
 // --------------------------------------------------------------------- dq ----
 template <typename T, int D, int MODE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, (D <= 128 ? 2 : 1))
 cmpattn_bwd_dq_kernel(CmpParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
@@ -612,7 +612,7 @@ static int attn_bwd_launch(const CmpParams& p, const SelBwdParams& kv, int batch
   {
     ProfScope ps_(MODE == CMP_MODE_WINDOW ? "winattn_bwd_dkdv_reduce" : "cmpattn_bwd_dkdv_reduce", stream);
     attn_bwd_dkdv_reduce_kernel<T, D, CMP_BK, KVM>
-        <<<dim3((unsigned)kv.max_blocks, hkv), 256, 0, stream>>>(kv);
+        <<<dim3((unsigned)kv.max_blocks, hkv, KV_REDUCE_SPLIT), 256, 0, stream>>>(kv);
   }
   return 0;
 }

@@ -8,12 +8,16 @@
 //   decode_topk_kernel: probabilities -> re-binned block scores -> top-k ids.
 //
 // Both attention modes are HBM-bound streams of K/V rows (g rows of queries
-// only), so one work-group per (request, kv head) lets its four waves take
-// 64-key tiles round-robin: K fragments go straight from global memory into
-// MFMA operands, the V tile is staged in a wave-private LDS region and read
-// back transposed, and the waves' partial (m, l, O) are merged through LDS.
-// The query heads occupy the first g of the 32 MFMA columns; column g carries
-// the scoring head.
+// only).  The keys of a (request, kv head) are split over work-groups of 512
+// keys so that the grid fills the chip whatever the cache lengths are; inside a
+// work-group the four waves take 32-key tiles round-robin: K fragments go
+// straight from global memory into 16x16x32 MFMA operands, the V tile is staged
+// in a wave-private LDS region and read back transposed.  The kernel is kept
+// lean in registers (several waves per SIMD keep enough loads in flight).  The
+// waves' partial (m, l, O) are merged through LDS into one fp32 partial per
+// work-group; a small merge kernel combines the partials of a request in a fixed
+// order.  The query heads occupy the first g of the 16 MFMA columns; column g
+// carries the scoring head.
 //
 // Semantics: fsa_preview/ops/compressed_attention_decode.py:361-490 (attention),
 // :494-592 (scores), :284-357 (transform), :203-205 (top-k);
@@ -24,7 +28,8 @@ namespace fsa {
 
 constexpr int DEC_MODE_COMPRESSED = 0;
 constexpr int DEC_MODE_SELECTED = 1;
-constexpr int DEC_TILE = 64;
+constexpr int DEC_TK = 32;    // keys per wave tile
+constexpr int DEC_TPS = 16;   // tiles per work-group (512 keys)
 
 struct DecParams {
   const void* q;   // [B, Hq, D]
@@ -41,192 +46,226 @@ struct DecParams {
   float* raw_score;         // compressed mode, optional: [Hkv, B, raw_ld] unscaled q.k of the scoring head
   int64_t raw_ld;
   int score_head_as_written;  // 0: first head of the group, 1: q-head with the kv head's own index
+  int max_keys;             // compressed mode: host upper bound of the visible keys of a request (more are ignored)
+  float* part;              // [B, Hkv, nsplit, g, 2 + D]: base-2 scaled max, sum, unnormalised O
+  int nsplit;
 };
 
 template <int D> struct DecLds {
-  static constexpr int VS = D + 16;
-  static constexpr int WAVE_BYTES = DEC_TILE * VS * 2;
-  static constexpr int MERGE_BYTES = 4 * ((D / 32) * 16 + 2) * 64 * 4;
+  static constexpr int VS = D + 8;
+  static constexpr int WAVE_BYTES = DEC_TK * VS * 2;
+  static constexpr int MERGE_BYTES = 4 * (D * 16 + 32) * 4;
   static constexpr int BYTES = 4 * WAVE_BYTES > MERGE_BYTES ? 4 * WAVE_BYTES : MERGE_BYTES;
 };
 
-template <typename T, int D, int MODE>
-__global__ void __launch_bounds__(256)
-decode_attn_kernel(DecParams p) {
-  typedef typename Elem<T>::vec8 vec8;
-  typedef typename Elem<T>::vec4 vec4;
-  constexpr int VS = DecLds<D>::VS;
-  constexpr int NA = DEC_TILE / 32, NKS = D / 16, NDT = D / 32, NJ = DEC_TILE / 16;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int b = blockIdx.x, h = blockIdx.y;
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int col = lane & 31, hh = lane >> 5;
-  T* Vs = reinterpret_cast<T*>(smem) + wv * (DEC_TILE * VS);
-
-  const int k0 = p.cu_k[b], len = p.cu_k[b + 1] - k0;
-  int n_tiles, n_keys = 0, tpb = 1;
+// number of 32-key tiles of request b (and, in compressed mode, its visible keys)
+template <int MODE>
+__device__ __forceinline__ int dec_tiles(const DecParams& p, int b, int len, int& n_keys, int& tpb) {
+  n_keys = 0;
+  tpb = 1;
   if (MODE == DEC_MODE_COMPRESSED) {
     const int qp = p.pos[b];
     n_keys = qp >= p.kernel_size - 1 ? min(len, (qp - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
-    n_tiles = (n_keys + DEC_TILE - 1) / DEC_TILE;
-  } else {
-    tpb = (p.block_size + DEC_TILE - 1) / DEC_TILE;
-    n_tiles = p.topk * tpb;
+    n_keys = min(n_keys, p.max_keys);
+    return (n_keys + DEC_TK - 1) / DEC_TK;
   }
+  tpb = (p.block_size + DEC_TK - 1) / DEC_TK;
+  return p.topk * tpb;
+}
+
+template <typename T, int D, int MODE>
+__global__ void __launch_bounds__(256, 2)
+decode_attn_kernel(DecParams p) {
+  typedef typename Elem<T>::vec8 vec8;
+  constexpr int VS = DecLds<D>::VS;
+  constexpr int NS = D / 32, NDT = D / 16, VCH = DEC_TK * (D / 8) / 64;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int split = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  const int l16 = lane & 15, kg = lane >> 4;
+  T* Vs = reinterpret_cast<T*>(smem) + wv * (DEC_TK * VS);
+
+  const int k0 = p.cu_k[b], len = p.cu_k[b + 1] - k0;
+  int n_keys, tpb;
+  const int n_tiles = dec_tiles<MODE>(p, b, len, n_keys, tpb);
+  const int t_lo = split * DEC_TPS;
+  if (t_lo >= n_tiles) return;  // the merge kernel derives the number of live splits the same way
+  const int t_hi = min(n_tiles, t_lo + DEC_TPS);
   const int32_t* sel = MODE == DEC_MODE_SELECTED ? p.topk_idx + ((int64_t)h * p.batch + b) * p.topk : nullptr;
 
-  // B operand: columns 0..g-1 = heads of the group, column g = scoring head (compressed mode)
-  vec8 qreg[NKS];
+  // B operand [k = d][n = column]: columns 0..g-1 = heads of the group, column g = scoring head (compressed mode)
+  vec8 qreg[NS];
   {
     int hq_i = -1;
-    if (col < p.g) hq_i = h * p.g + col;
-    else if (MODE == DEC_MODE_COMPRESSED && col == p.g) hq_i = p.score_head_as_written ? h : h * p.g;
-    const T* qrow = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)max(hq_i, 0) * p.q_sh + hh * (D / 2);
+    if (l16 < p.g) hq_i = h * p.g + l16;
+    else if (MODE == DEC_MODE_COMPRESSED && l16 == p.g) hq_i = p.score_head_as_written ? h : h * p.g;
+    const T* qrow = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)max(hq_i, 0) * p.q_sh + 8 * kg;
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) qreg[ks] = hq_i >= 0 ? load16<vec8>(qrow + ks * 8) : zero8<T>();
+    for (int s_ = 0; s_ < NS; ++s_) qreg[s_] = hq_i >= 0 ? load16<vec8>(qrow + 32 * s_) : zero8<T>();
   }
-  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh + hh * (D / 2);
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh + 8 * kg;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
-  const T* vtr = Vs + (4 * hh + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const T* vtr = Vs + (4 * kg + (l16 >> 2)) * VS + 4 * (l16 & 3);
 
-  float m = -INFINITY, l = 0.f;
-  f32x16 oacc[NDT];
+  float m = -INFINITY, l = 0.f;  // of column l16, replicated over the four key groups
+  f32x4 oacc[NDT];               // O^T[d = 16 t + 4 kg + i][column l16]
 #pragma unroll
-  for (int dt = 0; dt < NDT; ++dt)
+  for (int t = 0; t < NDT; ++t)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
+    for (int i = 0; i < 4; ++i) oacc[t][i] = 0.f;
 
-  for (int tt = wv; tt < n_tiles; tt += 4) {
+  for (int tt = t_lo + wv; tt < t_hi; tt += 4) {
     int row0, n_valid;
     if (MODE == DEC_MODE_COMPRESSED) {
-      row0 = tt * DEC_TILE;
-      n_valid = min(DEC_TILE, n_keys - row0);
+      row0 = tt * DEC_TK;
+      n_valid = min(DEC_TK, n_keys - row0);
     } else {
       const int t = tt / tpb, sub = tt - t * tpb;
       const int blk = sel[t];
       bool dup = false;
       for (int u = 0; u < t; ++u) dup |= sel[u] == blk;
-      row0 = blk * p.block_size + sub * DEC_TILE;
-      n_valid = (blk < 0 || dup) ? 0 : min(min(DEC_TILE, p.block_size - sub * DEC_TILE), len - row0);
+      row0 = blk * p.block_size + sub * DEC_TK;
+      n_valid = (blk < 0 || dup) ? 0 : min(min(DEC_TK, p.block_size - sub * DEC_TK), len - row0);
     }
     if (n_valid <= 0) continue;  // uniform per wave
-    // K fragments straight from global memory
-    f32x16 acc[NA];
+    // V rows (coalesced, 16 B per lane) are requested first so that they travel while S is computed
+    vec8 vst[VCH];
 #pragma unroll
-    for (int a = 0; a < NA; ++a) {
-      const int key = a * 32 + col;
+    for (int j = 0; j < VCH; ++j) {
+      const int c = lane + 64 * j, row = c / (D / 8), cc = c % (D / 8);
+      vst[j] = zero8<T>();  // rows past n_valid are zero so that 0 * garbage cannot appear
+      if (row < n_valid) vst[j] = load16<vec8>(vbase + (int64_t)(k0 + row0 + row) * p.v_sn + cc * 8);
+    }
+    // S^T[key][column] = K Q^T, K fragments straight from global memory
+    f32x4 acc[2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+      const int key = a * 16 + l16;
       const T* krow = kbase + (int64_t)(k0 + row0 + key) * p.k_sn;
-      vec8 kf[NKS];
+      vec8 kf[NS];
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) kf[ks] = key < n_valid ? load16<vec8>(krow + ks * 8) : zero8<T>();
+      for (int s_ = 0; s_ < NS; ++s_) kf[s_] = key < n_valid ? load16<vec8>(krow + 32 * s_) : zero8<T>();
 #pragma unroll
-      for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
+      for (int i = 0; i < 4; ++i) acc[a][i] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) acc[a] = Elem<T>::mfma32(kf[ks], qreg[ks], acc[a]);
+      for (int s_ = 0; s_ < NS; ++s_) acc[a] = Elem<T>::mfma16(kf[s_], qreg[s_], acc[a]);
     }
-    // V tile -> wave-private LDS (rows past n_valid are zero so that 0 * garbage cannot appear)
-    for (int c = lane; c < DEC_TILE * (D / 8); c += 64) {
-      const int row = c / (D / 8), cc = c % (D / 8);
-      vec8 x = zero8<T>();
-      if (row < n_valid) x = load16<vec8>(vbase + (int64_t)(k0 + row0 + row) * p.v_sn + cc * 8);
-      store16(&Vs[row * VS + cc * 8], x);
-    }
-    if (MODE == DEC_MODE_COMPRESSED && p.raw_score && col == p.g) {
+    if (MODE == DEC_MODE_COMPRESSED && p.raw_score && l16 == p.g) {
       float* rs = p.raw_score + ((int64_t)h * p.batch + b) * p.raw_ld + row0;
 #pragma unroll
-      for (int a = 0; a < NA; ++a)
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-          const int key0 = a * 32 + 8 * qd + 4 * hh;
-          if (row0 + key0 < p.raw_ld) {
-            f32x4 x;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x[e] = acc[a][4 * qd + e];
-            *reinterpret_cast<f32x4*>(rs + key0) = x;
-          }
-        }
+      for (int a = 0; a < 2; ++a) {
+        const int key0 = a * 16 + 4 * kg;
+        if (row0 + key0 < p.raw_ld) *reinterpret_cast<f32x4*>(rs + key0) = acc[a];
+      }
     }
     float mx = m;
 #pragma unroll
-    for (int a = 0; a < NA; ++a)
+    for (int a = 0; a < 2; ++a)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+      for (int i = 0; i < 4; ++i) {
+        const int key = a * 16 + 4 * kg + i;
         const float sv = key < n_valid ? acc[a][i] : -INFINITY;
         acc[a][i] = sv;
         mx = fmaxf(mx, sv);
       }
-    mx = fmaxf(mx, xor32(mx));
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float mref = mx * p.scale_log2;  // n_valid > 0, so mx is finite
     const float alpha = exp2f(m * p.scale_log2 - mref);
     float lsum = 0.f;
-    vec8 pk[NJ];
+    vec8 pk;  // contraction index 8 kg + j  <->  key 4 kg + j (j < 4), 16 + 4 kg + j - 4 (j >= 4)
 #pragma unroll
-    for (int a = 0; a < NA; ++a)
+    for (int a = 0; a < 2; ++a)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
+      for (int i = 0; i < 4; ++i) {
         const float pv = exp2f(acc[a][i] * p.scale_log2 - mref);
         lsum += pv;
-        pk[a * 2 + (i >> 3)][i & 7] = (T)pv;
+        pk[a * 4 + i] = (T)pv;
       }
-    lsum += xor32(lsum);
+    lsum += __shfl_xor(lsum, 16, 64);
+    lsum += __shfl_xor(lsum, 32, 64);
     l = l * alpha + lsum;
     m = mx;
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int c = lane + 64 * j, row = c / (D / 8), cc = c % (D / 8);
+      store16(&Vs[row * VS + cc * 8], vst[j]);
+    }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
+    for (int t = 0; t < NDT; ++t) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
-#pragma unroll
-      for (int j = 0; j < NJ; ++j) {
-        vec8 vf = lds_read_tr8<T>(vtr + 16 * j * VS + dt * 32, 8 * VS);
-        oacc[dt] = Elem<T>::mfma32(vf, pk[j], oacc[dt]);
-      }
+      for (int i = 0; i < 4; ++i) oacc[t][i] *= alpha;
+      vec8 vf = lds_read_tr8<T>(vtr + 16 * t, 16 * VS);  // V^T[d = 16 t + l16][keys in the order of pk]
+      oacc[t] = Elem<T>::mfma16(vf, pk, oacc[t]);
     }
     __builtin_amdgcn_wave_barrier();
   }
 
-  // merge the four waves' partial results: lane-wise, the accumulator layout is the same in every wave
+  // merge the four waves through LDS, then one fp32 partial per work-group
   __syncthreads();
   float* mg = reinterpret_cast<float*>(smem);
-  constexpr int PER = NDT * 16 + 2;
-  float* mine = mg + (wv * PER) * 64 + lane;
-  mine[0] = m;
-  mine[64] = l;
-#pragma unroll
-  for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) mine[(2 + dt * 16 + i) * 64] = oacc[dt][i];
-  __syncthreads();
-  if (wv != 0 || col >= p.g) return;
-  float mt = -INFINITY;
-#pragma unroll
-  for (int w = 0; w < 4; ++w) mt = fmaxf(mt, mg[(w * PER) * 64 + lane]);
-  float lt = 0.f, wgt[4];
-#pragma unroll
-  for (int w = 0; w < 4; ++w) {
-    const float mw = mg[(w * PER) * 64 + lane];
-    wgt[w] = mw == -INFINITY ? 0.f : exp2f((mw - mt) * p.scale_log2);
-    lt += wgt[w] * mg[(w * PER + 1) * 64 + lane];
+  constexpr int PER = D * 16 + 32;
+  float* mine = mg + wv * PER;
+  if (kg == 0) {
+    mine[l16] = m * p.scale_log2;
+    mine[16 + l16] = l;
   }
-  const float inv_l = lt > 0.f ? 1.f / lt : 0.f;
-  const int hq_i = h * p.g + col;
-  T* orow = reinterpret_cast<T*>(p.o) + ((int64_t)b * p.hq + hq_i) * D + 4 * hh;
 #pragma unroll
-  for (int dt = 0; dt < NDT; ++dt)
+  for (int t = 0; t < NDT; ++t)
 #pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-      vec4 x;
+    for (int i = 0; i < 4; ++i) mine[32 + (16 * t + 4 * kg + i) * 16 + l16] = oacc[t][i];
+  __syncthreads();
+  float* out = p.part + (((int64_t)b * p.hkv + h) * p.nsplit + split) * (p.g * (2 + D));
+  for (int e = tid; e < p.g * D; e += 256) {
+    const int col = e / D, d = e - col * D;
+    float mt = -INFINITY;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float s = 0.f;
+    for (int w = 0; w < 4; ++w) mt = fmaxf(mt, mg[w * PER + col]);
+    float lt = 0.f, o = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) s += wgt[w] * mg[(w * PER + 2 + dt * 16 + 4 * qd + e) * 64 + lane];
-        x[e] = (T)(s * inv_l);
-      }
-      store8(orow + dt * 32 + 8 * qd, x);
+    for (int w = 0; w < 4; ++w) {
+      const float mw = mg[w * PER + col];
+      const float wgt = mw == -INFINITY ? 0.f : exp2f(mw - mt);
+      lt += wgt * mg[w * PER + 16 + col];
+      o += wgt * mg[w * PER + 32 + d * 16 + col];
     }
-  if (hh == 0) p.lse[(int64_t)hq_i * p.batch + b] = lt > 0.f ? mt * p.scale_log2 + log2f(lt) : -INFINITY;
+    out[col * (2 + D) + 2 + d] = o;
+    if (d == 0) {
+      out[col * (2 + D)] = mt;
+      out[col * (2 + D) + 1] = lt;
+    }
+  }
+}
+
+// partials of a request -> o, lse (fixed order over the splits)
+template <typename T, int MODE>
+__global__ void __launch_bounds__(256)
+decode_merge_kernel(DecParams p, int D) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int len = p.cu_k[b + 1] - p.cu_k[b];
+  int n_keys, tpb;
+  const int n_tiles = dec_tiles<MODE>(p, b, len, n_keys, tpb);
+  const int ns = (n_tiles + DEC_TPS - 1) / DEC_TPS;
+  const int slot = p.g * (2 + D);
+  const float* part = p.part + ((int64_t)b * p.hkv + h) * p.nsplit * slot;
+  for (int e = threadIdx.x; e < p.g * D; e += 256) {
+    const int col = e / D, d = e - col * D;
+    const float* pc = part + col * (2 + D);
+    float mt = -INFINITY;
+    for (int s_ = 0; s_ < ns; ++s_) mt = fmaxf(mt, pc[s_ * slot]);
+    float lt = 0.f, o = 0.f;
+    for (int s_ = 0; s_ < ns; ++s_) {
+      const float ms = pc[s_ * slot];
+      const float wgt = ms == -INFINITY ? 0.f : exp2f(ms - mt);
+      lt += wgt * pc[s_ * slot + 1];
+      o += wgt * pc[s_ * slot + 2 + d];
+    }
+    const float inv_l = lt > 0.f ? 1.f / lt : 0.f;
+    const int hq_i = h * p.g + col;
+    reinterpret_cast<T*>(p.o)[((int64_t)b * p.hq + hq_i) * D + d] = (T)(o * inv_l);
+    if (d == 0) p.lse[(int64_t)hq_i * p.batch + b] = lt > 0.f ? mt + log2f(lt) : -INFINITY;
+  }
 }
 
 // ------------------------------------------------------------------ top-k ----
@@ -320,7 +359,8 @@ static int dec_launch(const DecParams& p, hipStream_t stream) {
     }
   }
   ProfScope ps_(MODE == DEC_MODE_COMPRESSED ? "decode_cmpattn" : "decode_selattn", stream);
-  decode_attn_kernel<T, D, MODE><<<dim3(p.batch, p.hkv), 256, lds, stream>>>(p);
+  if (p.nsplit > 0) decode_attn_kernel<T, D, MODE><<<dim3(p.nsplit, p.batch, p.hkv), 256, lds, stream>>>(p);
+  decode_merge_kernel<T, MODE><<<dim3(p.batch, p.hkv), 256, 0, stream>>>(p, D);
   return 0;
 }
 
@@ -339,9 +379,23 @@ static int dec_dispatch(int dtype, int head_dim, const DecParams& p, hipStream_t
   return FSA_ERR_UNSUPPORTED;
 }
 
+static int dec_splits(int64_t max_keys) {
+  const int64_t tiles = (max_keys + DEC_TK - 1) / DEC_TK;
+  return (int)((tiles + DEC_TPS - 1) / DEC_TPS);
+}
+static size_t dec_ws_bytes(int batch, int hq, int hkv, int d, int64_t max_keys) {
+  return (size_t)batch * hkv * (size_t)(dec_splits(max_keys) > 0 ? dec_splits(max_keys) : 1) * (hq / hkv) * (2 + d) * 4;
+}
+
 }  // namespace fsa
 
 using namespace fsa;
+
+extern "C" size_t fsa_decode_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                             int32_t head_dim, int64_t max_keys) {
+  if (batch < 1 || num_kv_heads < 1 || num_q_heads % num_kv_heads || max_keys < 0) return 0;
+  return dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_keys);
+}
 
 extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv, int32_t dtype,
                                   int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n,
@@ -349,14 +403,18 @@ extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv,
                                   const int32_t* cu_ck, const int32_t* pos, int32_t batch,
                                   int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                                   int32_t kernel_size, int32_t kernel_stride, float softmax_scale,
-                                  int32_t score_head_as_written, void* o, float* lse, float* raw_score,
-                                  int64_t raw_ld, void* stream_) {
+                                  int32_t score_head_as_written, int64_t max_keys, void* o, float* lse,
+                                  float* raw_score, int64_t raw_ld, void* workspace, size_t workspace_bytes,
+                                  void* stream_) {
   FSA_CHECK_ARG(q && ck && cv && cu_ck && pos && o && lse, "fsa_decode_cmpattn: null pointer");
   FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_decode_cmpattn: dtype must be bf16 or fp16");
   FSA_CHECK_ARG(num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
                 "fsa_decode_cmpattn: num_q_heads must be a multiple of num_kv_heads");
   const int g = num_q_heads / num_kv_heads;
-  FSA_CHECK_ARG(g <= 31, "fsa_decode_cmpattn: at most 31 query heads per kv head");
+  FSA_CHECK_ARG(g <= 15, "fsa_decode_cmpattn: at most 15 query heads per kv head");
+  FSA_CHECK_ARG(max_keys >= 0 && max_keys < (1ll << 30), "fsa_decode_cmpattn: bad max_keys");
+  FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_keys),
+                "fsa_decode_cmpattn: workspace too small (see fsa_decode_workspace_bytes)");
   FSA_CHECK_ARG(batch >= 1 && kernel_size >= 1 && kernel_stride >= 1, "fsa_decode_cmpattn: bad sizes");
   FSA_CHECK_ARG(!raw_score || (raw_ld >= 4 && raw_ld % 4 == 0), "fsa_decode_cmpattn: raw_ld must be a multiple of 4");
   FSA_CHECK_ARG(!score_head_as_written || num_kv_heads <= num_q_heads, "fsa_decode_cmpattn: bad scoring head");
@@ -367,6 +425,7 @@ extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv,
   p.kernel_size = kernel_size; p.kernel_stride = kernel_stride; p.scale_log2 = softmax_scale * LOG2E;
   p.o = o; p.lse = lse; p.raw_score = raw_score; p.raw_ld = raw_ld;
   p.score_head_as_written = score_head_as_written;
+  p.part = (float*)workspace; p.nsplit = dec_splits(max_keys); p.max_keys = (int)max_keys;
   int rc = dec_dispatch<DEC_MODE_COMPRESSED>(dtype, head_dim, p, (hipStream_t)stream_);
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_decode_cmpattn");
@@ -409,19 +468,23 @@ extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void
                                   const int32_t* cu_k, const int32_t* topk_idx, int32_t batch,
                                   int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                                   int32_t topk, int32_t block_size, float softmax_scale, void* o,
-                                  float* lse, void* stream_) {
+                                  float* lse, void* workspace, size_t workspace_bytes, void* stream_) {
   FSA_CHECK_ARG(q && k_cache && v_cache && cu_k && topk_idx && o && lse, "fsa_decode_selattn: null pointer");
   FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_decode_selattn: dtype must be bf16 or fp16");
   FSA_CHECK_ARG(num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
                 "fsa_decode_selattn: num_q_heads must be a multiple of num_kv_heads");
-  FSA_CHECK_ARG(num_q_heads / num_kv_heads <= 32, "fsa_decode_selattn: at most 32 query heads per kv head");
+  FSA_CHECK_ARG(num_q_heads / num_kv_heads <= 16, "fsa_decode_selattn: at most 16 query heads per kv head");
   FSA_CHECK_ARG(batch >= 1 && topk >= 1 && block_size >= 1, "fsa_decode_selattn: bad sizes");
+  const int64_t max_keys = (int64_t)topk * ((block_size + DEC_TK - 1) / DEC_TK) * DEC_TK;
+  FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_keys),
+                "fsa_decode_selattn: workspace too small (see fsa_decode_workspace_bytes)");
   DecParams p = {};
   p.q = q; p.k = k_cache; p.v = v_cache; p.q_sb = q_stride_b; p.q_sh = q_stride_h;
   p.k_sn = k_stride_n; p.k_sh = k_stride_h; p.v_sn = v_stride_n; p.v_sh = v_stride_h;
   p.cu_k = cu_k; p.topk_idx = topk_idx; p.batch = batch; p.hq = num_q_heads; p.hkv = num_kv_heads;
   p.g = num_q_heads / num_kv_heads; p.topk = topk; p.block_size = block_size;
   p.scale_log2 = softmax_scale * LOG2E; p.o = o; p.lse = lse;
+  p.part = (float*)workspace; p.nsplit = dec_splits(max_keys);
   int rc = dec_dispatch<DEC_MODE_SELECTED>(dtype, head_dim, p, (hipStream_t)stream_);
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_decode_selattn");

@@ -47,6 +47,7 @@ struct SelBwdParams {
 };
 
 
+constexpr int KV_REDUCE_SPLIT = 8;   // work-groups per block in the dK/dV reduce kernel
 constexpr int KV_MODE_SELECTED = 0;
 constexpr int KV_MODE_COMPRESSED = 1;
 constexpr int KV_MODE_WINDOW = 2;  // sliding window: key p visible to query i iff i - window <= p <= i
@@ -431,7 +432,8 @@ attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
   if (nt == 1) return;
   KvBlock<MODE, BK> blk;
   blk.init(p, gb);
-  for (int c = threadIdx.x; c < BK * (D / 4); c += 256) {
+  // gridDim.z work-groups share one block: the sum over its partials is a chain of dependent loads
+  for (int c = blockIdx.z * 256 + threadIdx.x; c < BK * (D / 4); c += 256 * gridDim.z) {
     const int key = c / (D / 4), d4 = (c % (D / 4)) * 4;
     const int tok = blk.key_row0 + key;
     if (key >= blk.n_keys_valid) continue;

@@ -62,12 +62,13 @@ SIGNATURES = {
                                           vp, vp, vp]),
     "fsa_linear_compress_bwd": (C.c_int, [vp, vp, vp, vp, i32, i64, i64, vp, vp, i32, i64, i64, i32, i32,
                                           i32, i32, vp, vp, vp, vp, vp]),
+    "fsa_decode_workspace_bytes": (C.c_size_t, [i32, i32, i32, i32, i64]),
     "fsa_decode_cmpattn": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp,
-                                     i32, i32, i32, i32, i32, i32, f32, i32, vp, vp, vp, i64, vp]),
+                                     i32, i32, i32, i32, i32, i32, f32, i32, i64, vp, vp, vp, i64, vp, sz, vp]),
     "fsa_decode_topk": (C.c_int, [vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                   i32, i32, i32, i32, f32, i64, vp, vp, vp]),
     "fsa_decode_selattn": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp,
-                                     i32, i32, i32, i32, i32, i32, f32, vp, vp, vp]),
+                                     i32, i32, i32, i32, i32, i32, f32, vp, vp, vp, sz, vp]),
 }
 
 

@@ -251,11 +251,14 @@ def decode_cmpattn(q, ck, cv, cu_ck, pos, kernel_size, kernel_stride, max_ck, so
     lse = torch.empty((hq, b), dtype=torch.float32, device=dev)
     ld = (max(int(max_ck), 1) + 3) // 4 * 4
     raw = torch.empty((hkv, b, ld), dtype=torch.float32, device=dev) if want_scores else None
+    max_keys = max(int(max_ck), 0)
+    ws_bytes = max(256, lib.fsa_decode_workspace_bytes(b, hq, hkv, d, max_keys))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     rc = lib.fsa_decode_cmpattn(_ptr(q), _ptr(ck), _ptr(cv), _DTYPE[q.dtype], q.stride(0), q.stride(1),
                                 ck.stride(0), ck.stride(1), cv.stride(0), cv.stride(1), _ptr(cu_ck), _ptr(pos),
                                 b, hq, hkv, d, kernel_size, kernel_stride, float(softmax_scale),
-                                1 if score_head_as_written else 0, _ptr(o), _ptr(lse), _ptr(raw), ld,
-                                _stream(dev))
+                                1 if score_head_as_written else 0, max_keys, _ptr(o), _ptr(lse), _ptr(raw), ld,
+                                _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_decode_cmpattn")
     return o, lse, raw
 
@@ -293,10 +296,13 @@ def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scal
     dev = q.device
     o = torch.empty((b, hq, d), dtype=q.dtype, device=dev)
     lse = torch.empty((hq, b), dtype=torch.float32, device=dev)
+    topk = topk_idx.shape[2]
+    ws_bytes = max(256, lib.fsa_decode_workspace_bytes(b, hq, hkv, d, topk * ((block_size + 31) // 32) * 32))
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     rc = lib.fsa_decode_selattn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _DTYPE[q.dtype], q.stride(0), q.stride(1),
                                 k_cache.stride(0), k_cache.stride(1), v_cache.stride(0), v_cache.stride(1),
                                 _ptr(cu_k), _ptr(topk_idx), b, hq, hkv, d, topk_idx.shape[2], block_size,
-                                float(softmax_scale), _ptr(o), _ptr(lse), _stream(dev))
+                                float(softmax_scale), _ptr(o), _ptr(lse), _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_decode_selattn")
     return o, lse
 

@@ -225,14 +225,26 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
  * (fsa_preview/ops/selected_attention_decode.py:8-42): the g heads of a group
  * attend every cached key of the selected blocks (ids < 0, past the cache or
  * repeated are ignored).
+ *
+ * Both attention calls split the keys of a request over several work-groups
+ * and merge their fp32 partials in a fixed order: the caller provides a
+ * workspace of fsa_decode_workspace_bytes(..., max_keys) bytes, max_keys being
+ * a host upper bound of the keys one request attends (compressed: the longest
+ * visible compressed cache, keys beyond it are ignored; selected: topk *
+ * block_size rounded up to 32-key tiles).  At most 15 (compressed) / 16
+ * (selected) query heads per kv head.
  * ---------------------------------------------------------------------- */
+size_t fsa_decode_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                  int32_t head_dim, int64_t max_keys);
+
 int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv, int32_t dtype,
                        int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
                        int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_ck, const int32_t* pos,
                        int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                        int32_t kernel_size, int32_t kernel_stride, float softmax_scale,
-                       int32_t score_head_as_written, void* o, float* lse, float* raw_score,
-                       int64_t raw_ld, void* stream);
+                       int32_t score_head_as_written, int64_t max_keys, void* o, float* lse,
+                       float* raw_score, int64_t raw_ld, void* workspace, size_t workspace_bytes,
+                       void* stream);
 
 int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const float* lse, const int32_t* cu_ck,
                     const int32_t* pos, const int32_t* seqlens, int32_t batch, int32_t num_q_heads,
@@ -246,7 +258,7 @@ int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, 
                        int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_k,
                        const int32_t* topk_idx, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
                        int32_t head_dim, int32_t topk, int32_t block_size, float softmax_scale, void* o,
-                       float* lse, void* stream);
+                       float* lse, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------
  * Sliding-window attention: the query at sequence-local position i attends the
