@@ -291,6 +291,72 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
     }
 }
 
+// -------------------------------------------------------------- gate merge ----
+// out[n, :] = g[n,0] a[n, :] + g[n,1] b[n, :] + g[n,2] c[n, :]  (one wave per token row, 16-byte chunks,
+// fp32 sum rounded once); backward: d_a = g0 d_out (same for b, c) and d_g[n,i] = <d_out[n, :], x_i[n, :]>.
+template <typename T>
+__global__ void __launch_bounds__(256)
+gate_merge_fwd_kernel(const T* __restrict__ a, const T* __restrict__ b, const T* __restrict__ c,
+                      const T* __restrict__ gate, T* __restrict__ out, int64_t n_tokens, int row) {
+  typedef typename Elem<T>::vec8 vec8;
+  const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= n_tokens) return;
+  const int lane = threadIdx.x & 63;
+  const float g0 = (float)gate[n * 3], g1 = (float)gate[n * 3 + 1], g2 = (float)gate[n * 3 + 2];
+  const int64_t base = n * row;
+  for (int e = lane * 8; e < row; e += 512) {
+    const vec8 x = load16<vec8>(a + base + e), y = load16<vec8>(b + base + e), z = load16<vec8>(c + base + e);
+    vec8 r;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = (T)(g0 * (float)x[i] + g1 * (float)y[i] + g2 * (float)z[i]);
+    store16(out + base + e, r);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+gate_merge_bwd_kernel(const T* __restrict__ d_out, const T* __restrict__ a, const T* __restrict__ b,
+                      const T* __restrict__ c, const T* __restrict__ gate, T* __restrict__ d_a,
+                      T* __restrict__ d_b, T* __restrict__ d_c, T* __restrict__ d_gate, int64_t n_tokens,
+                      int row) {
+  typedef typename Elem<T>::vec8 vec8;
+  const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= n_tokens) return;
+  const int lane = threadIdx.x & 63;
+  const float g0 = (float)gate[n * 3], g1 = (float)gate[n * 3 + 1], g2 = (float)gate[n * 3 + 2];
+  const int64_t base = n * row;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f;
+  for (int e = lane * 8; e < row; e += 512) {
+    const vec8 w = load16<vec8>(d_out + base + e);
+    const vec8 x = load16<vec8>(a + base + e), y = load16<vec8>(b + base + e), z = load16<vec8>(c + base + e);
+    vec8 ra, rb, rc;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float wf = (float)w[i];
+      s0 += wf * (float)x[i];
+      s1 += wf * (float)y[i];
+      s2 += wf * (float)z[i];
+      ra[i] = (T)(g0 * wf);
+      rb[i] = (T)(g1 * wf);
+      rc[i] = (T)(g2 * wf);
+    }
+    store16(d_a + base + e, ra);
+    store16(d_b + base + e, rb);
+    store16(d_c + base + e, rc);
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) {
+    s0 += __shfl_xor(s0, o, 64);
+    s1 += __shfl_xor(s1, o, 64);
+    s2 += __shfl_xor(s2, o, 64);
+  }
+  if (lane == 0) {
+    d_gate[n * 3] = (T)s0;
+    d_gate[n * 3 + 1] = (T)s1;
+    d_gate[n * 3 + 2] = (T)s2;
+  }
+}
+
 }  // namespace fsa
 
 using namespace fsa;
@@ -415,5 +481,47 @@ extern "C" int fsa_linear_compress_bwd(const void* x, const void* w, const void*
     lc_bwd_t<_Float16>(x, x_stride_n, x_stride_h, w, pe, dy, cu_seqlens_x, cu_seqlens_y, batch, max_seqlen_x,
                        total_y, num_heads, head_dim, kernel_size, kernel_stride, dx, dw, dpe, dbias_scratch, stream);
   FSA_CHECK_LAUNCH("fsa_linear_compress_bwd");
+  return 0;
+}
+
+extern "C" int fsa_gate_merge_fwd(const void* a, const void* b, const void* c, const void* gate, int32_t dtype,
+                                  int64_t total_tokens, int32_t row_elems, void* out, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FSA_CHECK_ARG(a && b && c && gate && out, "fsa_gate_merge_fwd: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_gate_merge_fwd: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(row_elems >= 8 && row_elems % 8 == 0, "fsa_gate_merge_fwd: row_elems must be a multiple of 8");
+  if (total_tokens <= 0) return 0;
+  const unsigned grid = (unsigned)((total_tokens + 3) / 4);
+  ProfScope ps_("gate_merge_fwd", stream);
+  if (dtype == FSA_BF16)
+    gate_merge_fwd_kernel<__bf16><<<grid, 256, 0, stream>>>((const __bf16*)a, (const __bf16*)b, (const __bf16*)c,
+                                                            (const __bf16*)gate, (__bf16*)out, total_tokens, row_elems);
+  else
+    gate_merge_fwd_kernel<_Float16><<<grid, 256, 0, stream>>>((const _Float16*)a, (const _Float16*)b,
+                                                              (const _Float16*)c, (const _Float16*)gate,
+                                                              (_Float16*)out, total_tokens, row_elems);
+  FSA_CHECK_LAUNCH("fsa_gate_merge_fwd");
+  return 0;
+}
+
+extern "C" int fsa_gate_merge_bwd(const void* d_out, const void* a, const void* b, const void* c,
+                                  const void* gate, int32_t dtype, int64_t total_tokens, int32_t row_elems,
+                                  void* d_a, void* d_b, void* d_c, void* d_gate, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  FSA_CHECK_ARG(d_out && a && b && c && gate && d_a && d_b && d_c && d_gate, "fsa_gate_merge_bwd: null pointer");
+  FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_gate_merge_bwd: dtype must be bf16 or fp16");
+  FSA_CHECK_ARG(row_elems >= 8 && row_elems % 8 == 0, "fsa_gate_merge_bwd: row_elems must be a multiple of 8");
+  if (total_tokens <= 0) return 0;
+  const unsigned grid = (unsigned)((total_tokens + 3) / 4);
+  ProfScope ps_("gate_merge_bwd", stream);
+  if (dtype == FSA_BF16)
+    gate_merge_bwd_kernel<__bf16><<<grid, 256, 0, stream>>>(
+        (const __bf16*)d_out, (const __bf16*)a, (const __bf16*)b, (const __bf16*)c, (const __bf16*)gate,
+        (__bf16*)d_a, (__bf16*)d_b, (__bf16*)d_c, (__bf16*)d_gate, total_tokens, row_elems);
+  else
+    gate_merge_bwd_kernel<_Float16><<<grid, 256, 0, stream>>>(
+        (const _Float16*)d_out, (const _Float16*)a, (const _Float16*)b, (const _Float16*)c, (const _Float16*)gate,
+        (_Float16*)d_a, (_Float16*)d_b, (_Float16*)d_c, (_Float16*)d_gate, total_tokens, row_elems);
+  FSA_CHECK_LAUNCH("fsa_gate_merge_bwd");
   return 0;
 }

@@ -33,6 +33,20 @@ class _SlidingWindowAttention(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
+class _GateMerge(torch.autograd.Function):
+    """Gate-weighted sum of the three branch outputs in one pass (fsa/module/fsa.py:162-167)."""
+
+    @staticmethod
+    def forward(ctx, a, b, c, gate):
+        ctx.save_for_backward(a, b, c, gate)
+        return _ops.gate_merge_fwd(a, b, c, gate)
+
+    @staticmethod
+    def backward(ctx, d_out):
+        a, b, c, gate = ctx.saved_tensors
+        return _ops.gate_merge_bwd(d_out, a, b, c, gate)
+
+
 class FlashSparseAttention(torch.nn.Module):
     def __init__(
         self,
@@ -123,11 +137,7 @@ class FlashSparseAttention(torch.nn.Module):
         sliding_attn_output = _SlidingWindowAttention.apply(q, k, v, cu_seqlens, max_len, self.window_size)
 
         gate = self.gate(x)
-        attn_output = (
-            gate[:, 0:1, None] * compressed_attn_output
-            + gate[:, 1:2, None] * sparse_attn_output
-            + gate[:, 2:3, None] * sliding_attn_output
-        )
+        attn_output = _GateMerge.apply(compressed_attn_output, sparse_attn_output, sliding_attn_output, gate)
         attn_output = self.proj_o(attn_output.reshape(attn_output.shape[0], -1))
         if return_topk_idx:
             return attn_output, topk_idx

@@ -62,6 +62,8 @@ SIGNATURES = {
                                           vp, vp, vp]),
     "fsa_linear_compress_bwd": (C.c_int, [vp, vp, vp, vp, i32, i64, i64, vp, vp, i32, i64, i64, i32, i32,
                                           i32, i32, vp, vp, vp, vp, vp]),
+    "fsa_gate_merge_fwd": (C.c_int, [vp, vp, vp, vp, i32, i64, i32, vp, vp]),
+    "fsa_gate_merge_bwd": (C.c_int, [vp, vp, vp, vp, vp, i32, i64, i32, vp, vp, vp, vp, vp]),
     "fsa_decode_workspace_bytes": (C.c_size_t, [i32, i32, i32, i32, i64]),
     "fsa_decode_cmpattn": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp,
                                      i32, i32, i32, i32, i32, i32, f32, i32, i64, vp, vp, vp, i64, vp, sz, vp]),

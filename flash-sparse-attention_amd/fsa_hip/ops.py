@@ -403,3 +403,31 @@ def linear_compress_bwd(x, w, dy, cu_x, cu_y, max_x, kernel_size, kernel_stride,
                                      _ptr(dbias), _stream(dev))
     _lib.check(rc, "fsa_linear_compress_bwd")
     return dx, dw, dpe
+
+
+def gate_merge_fwd(a, b, c, gate):
+    """out = gate[:,0] a + gate[:,1] b + gate[:,2] c for a, b, c [N, H, D] and gate [N, 3], one pass."""
+    _require_cuda(a, b, c, gate)
+    assert a.dtype in _DTYPE and a.dtype == b.dtype == c.dtype == gate.dtype
+    assert a.shape == b.shape == c.shape and gate.shape == (a.shape[0], 3)
+    a, b, c, gate = (t.contiguous() for t in (a, b, c, gate))
+    n = a.shape[0]
+    row = a.numel() // max(n, 1)
+    out = torch.empty_like(a)
+    rc = _lib.load().fsa_gate_merge_fwd(_ptr(a), _ptr(b), _ptr(c), _ptr(gate), _DTYPE[a.dtype], n, row, _ptr(out),
+                                        _stream(a.device))
+    _lib.check(rc, "fsa_gate_merge_fwd")
+    return out
+
+
+def gate_merge_bwd(d_out, a, b, c, gate):
+    """(d_a, d_b, d_c, d_gate) of gate_merge_fwd."""
+    _require_cuda(d_out, a, b, c, gate)
+    d_out, a, b, c, gate = (t.contiguous() for t in (d_out, a, b, c, gate))
+    n = a.shape[0]
+    row = a.numel() // max(n, 1)
+    d_a, d_b, d_c, d_gate = torch.empty_like(a), torch.empty_like(b), torch.empty_like(c), torch.empty_like(gate)
+    rc = _lib.load().fsa_gate_merge_bwd(_ptr(d_out), _ptr(a), _ptr(b), _ptr(c), _ptr(gate), _DTYPE[a.dtype], n, row,
+                                        _ptr(d_a), _ptr(d_b), _ptr(d_c), _ptr(d_gate), _stream(a.device))
+    _lib.check(rc, "fsa_gate_merge_bwd")
+    return d_a, d_b, d_c, d_gate

@@ -324,6 +324,22 @@ int fsa_linear_compress_bwd(const void* x, const void* w, const void* pe, const 
                             int32_t num_heads, int32_t head_dim, int32_t kernel_size, int32_t kernel_stride,
                             void* dx, void* dw, void* dpe, float* dbias_scratch, void* stream);
 
+/* ------------------------------------------------------------------------
+ * Gate-weighted merge of the three branch outputs, one pass:
+ *   out[n, :] = gate[n,0] a[n, :] + gate[n,1] b[n, :] + gate[n,2] c[n, :]
+ * a, b, c, out contiguous [N, row_elems] (row_elems = Hq*D), gate contiguous
+ * [N, 3] (already passed through the sigmoid), all in `dtype`; fp32 sum, one
+ * rounding.  Backward: d_a = gate[n,0] d_out (same for b, c), d_gate[n,i] =
+ * <d_out[n, :], x_i[n, :]>.  Replaces the broadcast multiply-adds of
+ * fsa/module/fsa.py:162-167 (five elementwise passes forward, nine backward).
+ * ---------------------------------------------------------------------- */
+int fsa_gate_merge_fwd(const void* a, const void* b, const void* c, const void* gate, int32_t dtype,
+                       int64_t total_tokens, int32_t row_elems, void* out, void* stream);
+
+int fsa_gate_merge_bwd(const void* d_out, const void* a, const void* b, const void* c, const void* gate,
+                       int32_t dtype, int64_t total_tokens, int32_t row_elems, void* d_a, void* d_b,
+                       void* d_c, void* d_gate, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

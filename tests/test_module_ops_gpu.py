@@ -78,3 +78,23 @@ def test_linear_compress_fwd_bwd(dev, cu, h, d, ks, st, dtype, with_pe):
               f"(ref max {ref.abs().max().item():.2f})", flush=True)
         assert rel < 3 * ulp, name
         assert excess <= (2e-2 if dtype == torch.bfloat16 else 5e-3), name
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gate_merge(dev, dtype):
+    """One-pass gate-weighted merge and its backward against the fp32 formulas (one output rounding)."""
+    gen = torch.Generator().manual_seed(9)
+    n, h, d = 1003, 6, 128
+    a, b, c, w = (torch.randn(n, h, d, generator=gen).to(dtype) for _ in range(4))
+    gate = torch.sigmoid(torch.randn(n, 3, generator=gen)).to(dtype)
+    out = ops.gate_merge_fwd(a.to(dev), b.to(dev), c.to(dev), gate.to(dev))
+    d_a, d_b, d_c, d_g = ops.gate_merge_bwd(w.to(dev), a.to(dev), b.to(dev), c.to(dev), gate.to(dev))
+    torch.cuda.synchronize()
+    g32 = gate.float()
+    ref = g32[:, 0, None, None] * a.float() + g32[:, 1, None, None] * b.float() + g32[:, 2, None, None] * c.float()
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    assert ((out.float().cpu() - ref).abs() <= ulp * ref.abs() + 1e-6).all()   # fp32 sum (fused multiply-adds), one rounding
+    for i, (got, x) in enumerate(((d_a, a), (d_b, b), (d_c, c))):
+        assert torch.equal(got.cpu(), (g32[:, i, None, None] * w.float()).to(dtype))
+        dg = (w.float() * x.float()).sum((1, 2))
+        assert torch.allclose(d_g[:, i].float().cpu(), dg, rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10, atol=1e-2)
