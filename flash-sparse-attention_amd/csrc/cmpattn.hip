@@ -165,7 +165,7 @@ cmpattn_fwd_kernel(CmpParams p) {
     for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float pv = exp2f(acc[a][i] * p.scale_log2 - mref);
+        const float pv = fast_exp2(acc[a][i] * p.scale_log2 - mref);
         lsum += pv;
         pk[a * 2 + (i >> 3)][i & 7] = (T)pv;
       }
@@ -277,7 +277,7 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-        const float pv = (key <= limit && key >= limit_lo) ? exp2f(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
+        const float pv = (key <= limit && key >= limit_lo) ? fast_exp2(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
         dsk[a * 2 + (i >> 3)][i & 7] = (T)(pv * (dp[a][i] - delta_r) * p.scale);
       }
 #pragma unroll
@@ -436,7 +436,7 @@ cmp_score_kernel(CmpParams p) {
             f32x4 x;
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              x[e] = key0 + e <= limit ? exp2f(acc[a][4 * qd + e] * p.scale_log2 - lse_r) : 0.f;
+              x[e] = key0 + e <= limit ? fast_exp2(acc[a][4 * qd + e] * p.scale_log2 - lse_r) : 0.f;
             *reinterpret_cast<f32x4*>(srow + jt + key0) = x;
           }
         }

@@ -178,7 +178,7 @@ decode_attn_kernel(DecParams p) {
     for (int a = 0; a < 2; ++a)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float pv = exp2f(acc[a][i] * p.scale_log2 - mref);
+        const float pv = fast_exp2(acc[a][i] * p.scale_log2 - mref);
         lsum += pv;
         pk[a * 4 + i] = (T)pv;
       }
@@ -308,7 +308,7 @@ decode_topk_kernel(DecTopkParams p) {
       const int c = c0 + o;
       if (c >= 0 && c < n_vis) {
         const int wgt = min(min(o, n_off - 1 - o), min(na, ne) - 1) + 1;
-        acc += (float)wgt * exp2f(rs[c] * p.scale_log2 - lse_r);
+        acc += (float)wgt * fast_exp2(rs[c] * p.scale_log2 - lse_r);
       }
     }
     if (blk < p.init_blocks || (bq >= blk && bq < blk + p.local_blocks)) acc = INFINITY;

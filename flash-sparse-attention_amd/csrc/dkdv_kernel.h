@@ -313,7 +313,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const bool vis = key <= lim_r[i] && (MODE != KV_MODE_WINDOW || key >= llo_r[i]);
-        const float pv = vis ? exp2f(sacc[i] * p.scale_log2 - lse_r[i]) : 0.f;
+        const float pv = vis ? fast_exp2(sacc[i] * p.scale_log2 - lse_r[i]) : 0.f;
         const float ds = pv * (dpacc[i] - del_r[i]) * p.scale;
         pk[rt][i] = (T)pv;
         dsk[rt][i] = (T)ds;

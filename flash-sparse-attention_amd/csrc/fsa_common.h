@@ -89,6 +89,10 @@ __device__ __forceinline__ typename Elem<T>::vec8 lds_read_tr8(const T* p, int s
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// 2^x by the hardware instruction alone (1 ulp; results below 2^-126 flush to zero, -inf gives 0): the
+// library exp2f adds a denormal-range rescaling that costs several VALU operations per element
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
 // largest i in [0, n) with a[i] <= x, for ascending a[0..n) with a[0] <= x

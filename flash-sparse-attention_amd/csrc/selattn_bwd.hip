@@ -151,7 +151,7 @@ selattn_bwd_dq_kernel(SelBwdParams p) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-        const float pv = key <= limit ? exp2f(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
+        const float pv = key <= limit ? fast_exp2(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
         const float ds = pv * (dp[a][i] - delta_r) * p.scale;
         dsk[a * 2 + (i >> 3)][i & 7] = (T)ds;
       }

@@ -183,7 +183,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
     for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float pv = exp2f(acc[a][i] * p.scale_log2 - mref);
+        const float pv = fast_exp2(acc[a][i] * p.scale_log2 - mref);
         l += pv;
         pk[a * 2 + (i >> 3)][i & 7] = (T)pv;
       }
