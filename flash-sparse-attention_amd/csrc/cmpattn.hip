@@ -612,7 +612,7 @@ static int attn_bwd_launch(const CmpParams& p, const SelBwdParams& kv, int batch
   {
     ProfScope ps_(MODE == CMP_MODE_WINDOW ? "winattn_bwd_dkdv_reduce" : "cmpattn_bwd_dkdv_reduce", stream);
     attn_bwd_dkdv_reduce_kernel<T, D, CMP_BK, KVM>
-        <<<dim3((unsigned)kv.max_blocks, hkv, KV_REDUCE_SPLIT), 256, 0, stream>>>(kv);
+        <<<dim3((unsigned)((kv.max_blocks + KV_REDUCE_SPAN - 1) / KV_REDUCE_SPAN), hkv, KV_REDUCE_SPLIT), 256, 0, stream>>>(kv);
   }
   return 0;
 }

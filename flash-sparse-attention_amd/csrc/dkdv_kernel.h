@@ -47,7 +47,8 @@ struct SelBwdParams {
 };
 
 
-constexpr int KV_REDUCE_SPLIT = 8;   // work-groups per block in the dK/dV reduce kernel
+constexpr int KV_REDUCE_SPLIT = 32;  // work-groups that share the blocks of one span in the dK/dV reduce kernel
+constexpr int KV_REDUCE_SPAN = 64;   // blocks examined by one work-group of that kernel
 constexpr int KV_MODE_SELECTED = 0;
 constexpr int KV_MODE_COMPRESSED = 1;
 constexpr int KV_MODE_WINDOW = 2;  // sliding window: key p visible to query i iff i - window <= p <= i
@@ -425,32 +426,63 @@ __global__ void __launch_bounds__(256)
 attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
   typedef typename Elem<T>::vec4 vec4;
   const int h = blockIdx.y;
-  const int gb = blockIdx.x;
-  if (gb >= p.cu_blocks[p.batch]) return;
   const int32_t* tp = p.tile_prefix + h * (p.max_blocks + 1);
-  const int t0 = tp[gb], nt = tp[gb + 1] - t0;
-  if (nt == 1) return;
-  KvBlock<MODE, BK> blk;
-  blk.init(p, gb);
-  // gridDim.z work-groups share one block: the sum over its partials is a chain of dependent loads
-  for (int c = blockIdx.z * 256 + threadIdx.x; c < BK * (D / 4); c += 256 * gridDim.z) {
-    const int key = c / (D / 4), d4 = (c % (D / 4)) * 4;
-    const int tok = blk.key_row0 + key;
-    if (key >= blk.n_keys_valid) continue;
-    f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = {0.f, 0.f, 0.f, 0.f};
-    for (int t = 0; t < nt; ++t) {
-      const float* part = p.dkdv_part + ((int64_t)h * p.max_tiles + t0 + t) * (2 * BK * D) + key * D + d4;
-      sk += *reinterpret_cast<const f32x4*>(part);
-      sv += *reinterpret_cast<const f32x4*>(part + BK * D);
-    }
-    vec4 a, b;
+  const int n_blocks = p.cu_blocks[p.batch];
+  // a work-group looks at KV_REDUCE_SPAN blocks at once: almost all of them have a single tile, whose
+  // work-group wrote dK / dV itself
+  __shared__ int todo[KV_REDUCE_SPAN];
+  __shared__ int n_todo;
+  const int gb0 = blockIdx.x * KV_REDUCE_SPAN;
+  if (threadIdx.x < WAVE) {
+    static_assert(KV_REDUCE_SPAN == WAVE, "one lane per block of the span");
+    const int gbi = gb0 + threadIdx.x;
+    const bool multi = gbi < n_blocks && tp[gbi + 1] - tp[gbi] != 1;  // no tile at all: zeros
+    const uint64_t m = __ballot(multi);
+    if (multi) todo[__popcll(m & ((1ull << threadIdx.x) - 1))] = gbi;
+    if (threadIdx.x == 0) n_todo = __popcll(m);
+  }
+  __syncthreads();
+  // unit of work: 256 consecutive (key, 4 dims) items of one block; the gridDim.z work-groups of the span
+  // take the units round-robin
+  constexpr int CH = BK * (D / 4) / 256;
+  for (int u_ = blockIdx.z; u_ < n_todo * CH; u_ += gridDim.z) {
+    const int gb = todo[u_ / CH];
+    const int t0 = tp[gb], nt = tp[gb + 1] - t0;
+    KvBlock<MODE, BK> blk;
+    blk.init(p, gb);
+    {
+      const int c = (u_ % CH) * 256 + threadIdx.x;
+      const int key = c / (D / 4), d4 = (c % (D / 4)) * 4;
+      const int tok = blk.key_row0 + key;
+      if (key >= blk.n_keys_valid) continue;
+      f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = {0.f, 0.f, 0.f, 0.f};
+      const float* part0 = p.dkdv_part + ((int64_t)h * p.max_tiles + t0) * (2 * BK * D) + key * D + d4;
+      // the loads of a batch are issued together (one memory latency per batch), the adds keep the tile order
+      constexpr int UB = 8;
+      for (int tb = 0; tb < nt; tb += UB) {
+        f32x4 xk[UB], xv[UB];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      a[i] = (T)sk[i];
-      b[i] = (T)sv[i];
+        for (int u = 0; u < UB; ++u) {
+          const float* part = part0 + (int64_t)max(min(tb + u, nt - 1), 0) * (2 * BK * D);
+          xk[u] = *reinterpret_cast<const f32x4*>(part);
+          xv[u] = *reinterpret_cast<const f32x4*>(part + BK * D);
+        }
+#pragma unroll
+        for (int u = 0; u < UB; ++u)
+          if (tb + u < nt) {
+            sk += xk[u];
+            sv += xv[u];
+          }
+      }
+      vec4 a, b;
+#pragma unroll
+      for (int i2 = 0; i2 < 4; ++i2) {
+        a[i2] = (T)sk[i2];
+        b[i2] = (T)sv[i2];
+      }
+      store8(reinterpret_cast<T*>(p.dk) + (int64_t)tok * p.dk_sn + (int64_t)h * p.dk_sh + d4, a);
+      store8(reinterpret_cast<T*>(p.dv) + (int64_t)tok * p.dk_sn + (int64_t)h * p.dk_sh + d4, b);
     }
-    store8(reinterpret_cast<T*>(p.dk) + (int64_t)tok * p.dk_sn + (int64_t)h * p.dk_sh + d4, a);
-    store8(reinterpret_cast<T*>(p.dv) + (int64_t)tok * p.dk_sn + (int64_t)h * p.dk_sh + d4, b);
   }
 }
 

@@ -295,7 +295,7 @@ static int launch_bwd(const SelBwdParams& pdq, const SelBwdParams& pkv, int hkv,
   }
   {
     ProfScope ps_("selattn_bwd_dkdv_reduce", stream);
-    attn_bwd_dkdv_reduce_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3((unsigned)pkv.max_blocks, hkv, KV_REDUCE_SPLIT), 256, 0, stream>>>(pkv);
+    attn_bwd_dkdv_reduce_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3((unsigned)((pkv.max_blocks + KV_REDUCE_SPAN - 1) / KV_REDUCE_SPAN), hkv, KV_REDUCE_SPLIT), 256, 0, stream>>>(pkv);
   }
   return 0;
 }
