@@ -80,7 +80,9 @@ decode_attn_kernel(DecParams p) {
   constexpr int VS = DecLds<D>::VS;
   constexpr int NS = D / 32, NDT = D / 16, VCH = DEC_TK * (D / 8) / 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  const int split = blockIdx.x, b = blockIdx.y, h = blockIdx.z;
+  // kv heads vary fastest over the grid: work-groups that run together read neighbouring 2*D-byte pieces of the
+  // same cache rows
+  const int h = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int l16 = lane & 15, kg = lane >> 4;
   T* Vs = reinterpret_cast<T*>(smem) + wv * (DEC_TK * VS);
@@ -285,11 +287,16 @@ struct DecTopkParams {
   int64_t score_ld;
 };
 
-// one wave per (request, kv head)
-__global__ void __launch_bounds__(64)
+// one work-group per (request, kv head): the block scores stay in LDS, every selection round is an arg-max
+// over the work-group (value first, lower block id on equal values)
+constexpr int DEC_TOPK_THREADS = 256;
+
+__global__ void __launch_bounds__(DEC_TOPK_THREADS)
 decode_topk_kernel(DecTopkParams p) {
   extern __shared__ float bs[];
-  const int b = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  __shared__ float wbest[DEC_TOPK_THREADS / WAVE];
+  __shared__ int wbest_id[DEC_TOPK_THREADS / WAVE];
+  const int b = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
   const int nc = p.cu_ck[b + 1] - p.cu_ck[b];
   const int qp = p.pos[b];
   const int n_vis = qp >= p.kernel_size - 1 ? min(nc, (qp - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
@@ -301,7 +308,7 @@ decode_topk_kernel(DecTopkParams p) {
   const int na = p.kernel_size / p.kernel_stride, ne = p.block_size / p.kernel_stride;
   const int n_off = na + ne - 1, pad = na - 1;
   const float* rs = p.raw_score + ((int64_t)h * p.batch + b) * p.raw_ld;
-  for (int blk = lane; blk < nblk; blk += 64) {
+  for (int blk = tid; blk < nblk; blk += DEC_TOPK_THREADS) {
     float acc = 0.f;
     const int c0 = blk * ne - pad;
     for (int o = 0; o < n_off; ++o) {
@@ -316,14 +323,14 @@ decode_topk_kernel(DecTopkParams p) {
     if (p.block_score) p.block_score[((int64_t)h * p.batch + b) * p.score_ld + blk] = acc;
   }
   if (p.block_score)
-    for (int64_t blk = nblk + lane; blk < p.score_ld; blk += 64)
+    for (int64_t blk = nblk + tid; blk < p.score_ld; blk += DEC_TOPK_THREADS)
       p.block_score[((int64_t)h * p.batch + b) * p.score_ld + blk] = -INFINITY;
-  __builtin_amdgcn_wave_barrier();
+  __syncthreads();
   int32_t* out = p.topk_idx + ((int64_t)h * p.batch + b) * p.topk;
   for (int t = 0; t < p.topk; ++t) {
     float best = -2.f;
     int best_id = 0x7fffffff;
-    for (int blk = lane; blk < nblk; blk += 64) {
+    for (int blk = tid; blk < nblk; blk += DEC_TOPK_THREADS) {  // ascending ids: the first maximum is kept
       const float vv = bs[blk];
       if (vv > best) {
         best = vv;
@@ -340,10 +347,26 @@ decode_topk_kernel(DecTopkParams p) {
       }
     }
     if (lane == 0) {
+      wbest[wv] = best;
+      wbest_id[wv] = best_id;
+    }
+    __syncthreads();
+    best = wbest[0];
+    best_id = wbest_id[0];
+#pragma unroll
+    for (int w = 1; w < DEC_TOPK_THREADS / WAVE; ++w) {
+      const float ov = wbest[w];
+      const int oi = wbest_id[w];
+      if (ov > best || (ov == best && oi < best_id)) {
+        best = ov;
+        best_id = oi;
+      }
+    }
+    if (tid == 0) {
       out[t] = best >= 0.f ? best_id : -1;  // fewer than topk blocks exist
       if (best >= 0.f) bs[best_id] = -1.f;
     }
-    __builtin_amdgcn_wave_barrier();
+    __syncthreads();
   }
 }
 
@@ -359,7 +382,7 @@ static int dec_launch(const DecParams& p, hipStream_t stream) {
     }
   }
   ProfScope ps_(MODE == DEC_MODE_COMPRESSED ? "decode_cmpattn" : "decode_selattn", stream);
-  if (p.nsplit > 0) decode_attn_kernel<T, D, MODE><<<dim3(p.nsplit, p.batch, p.hkv), 256, lds, stream>>>(p);
+  if (p.nsplit > 0) decode_attn_kernel<T, D, MODE><<<dim3(p.hkv, p.nsplit, p.batch), 256, lds, stream>>>(p);
   decode_merge_kernel<T, MODE><<<dim3(p.batch, p.hkv), 256, 0, stream>>>(p, D);
   return 0;
 }
@@ -456,7 +479,7 @@ extern "C" int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const flo
   p.score_ld = max_blocks;
   {
     ProfScope ps_("decode_topk", stream);
-    decode_topk_kernel<<<dim3(batch, num_kv_heads), 64, (size_t)max_blocks * 4, stream>>>(p);
+    decode_topk_kernel<<<dim3(batch, num_kv_heads), DEC_TOPK_THREADS, (size_t)max_blocks * 4, stream>>>(p);
   }
   FSA_CHECK_LAUNCH("fsa_decode_topk");
   return 0;
