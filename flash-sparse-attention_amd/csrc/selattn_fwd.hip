@@ -37,24 +37,33 @@ struct SelFwdParams {
   float* lse_part;
 };
 
-constexpr int SEL_THREADS = 256;
-constexpr int SEL_WG_ROWS = 128;                 // rows per pass of the 4 waves
-constexpr int SEL_TILE_ROWS = 8 * SEL_WG_ROWS;   // rows per work-group
+constexpr int SEL_TILE_ROWS = 1024;   // rows per work-group (4 or 8 passes of its waves)
 
 template <int D, int BK> struct SelLds {
   static constexpr int KS = D + 8;   // K row stride in elements (16 B pad: bank spread)
   static constexpr int VS = D + 16;  // V row stride in elements (32 B pad for the transposing reads)
   static constexpr int OS = D + 8;   // row stride of the per-wave output staging tile
-  static constexpr bool STAGE_OUT = (BK * KS + BK * VS + 4 * 32 * OS) * 2 <= 160 * 1024;
-  static constexpr int BYTES = (BK * KS + BK * VS + (STAGE_OUT ? 4 * 32 * OS : 0)) * 2;
-  static constexpr int MIN_WAVES = (D <= 128 && BK <= 64) ? 2 : 1;  // waves per SIMD the register budget allows
+  static constexpr int KV_BYTES = (BK * KS + BK * VS) * 2;
+  static constexpr int STAGE_BYTES = 32 * OS * 2;  // one wave's [32][D] tile
+  // Four waves with staging tiles, two work-groups per CU, where that fits in LDS.  Otherwise one work-group
+  // per CU: eight waves (two per SIMD) share the K / V copy, with staging tiles if LDS still holds them.
+  static constexpr bool TWO_WGS = KV_BYTES + 4 * STAGE_BYTES <= 80 * 1024;
+  static constexpr bool STAGE8 = KV_BYTES + 8 * STAGE_BYTES <= 160 * 1024;
+  static constexpr bool STAGE4 = KV_BYTES + 4 * STAGE_BYTES <= 160 * 1024;
+  static constexpr int THREADS = TWO_WGS ? 256 : (STAGE8 || !STAGE4) ? 512 : 256;
+  static constexpr int NWAVES = THREADS / 64;
+  static constexpr bool STAGE_OUT = KV_BYTES + NWAVES * STAGE_BYTES <= 160 * 1024;
+  static constexpr int BYTES = KV_BYTES + (STAGE_OUT ? NWAVES * STAGE_BYTES : 0);
+  static constexpr int WG_ROWS = NWAVES * 32;     // rows per pass of the work-group
+  static constexpr int MIN_WAVES = (THREADS == 256 && D <= 128 && BK <= 64) ? 2 : 1;  // waves per SIMD the register budget allows
 };
 
 template <typename T, int D, int BK>
-__global__ void __launch_bounds__(SEL_THREADS, (SelLds<D, BK>::MIN_WAVES))
+__global__ void __launch_bounds__((SelLds<D, BK>::THREADS), (SelLds<D, BK>::MIN_WAVES))
 selattn_fwd_main_kernel(SelFwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
   constexpr int KS = SelLds<D, BK>::KS, VS = SelLds<D, BK>::VS;
+  constexpr int SEL_THREADS = SelLds<D, BK>::THREADS, SEL_WG_ROWS = SelLds<D, BK>::WG_ROWS;
   constexpr int NA = BK / 32;   // S^T accumulators (32 keys each)
   constexpr int NKS = D / 16;   // k-steps of QK^T
   constexpr int NDT = D / 32;   // O^T accumulators (32 dims each)
@@ -331,7 +340,7 @@ static int launch_main(const SelFwdParams& p, int hkv, int64_t max_tiles, hipStr
   }
   dim3 grid((unsigned)max_tiles, hkv);
   ProfScope ps_("selattn_fwd_main", stream);
-  selattn_fwd_main_kernel<T, D, BK><<<grid, SEL_THREADS, lds, stream>>>(p);
+  selattn_fwd_main_kernel<T, D, BK><<<grid, SelLds<D, BK>::THREADS, lds, stream>>>(p);
   return 0;
 }
 
