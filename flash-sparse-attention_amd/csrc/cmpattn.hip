@@ -464,10 +464,14 @@ struct TopkParams {
 
 __device__ __forceinline__ float round_bf16(float x) { return (float)(__bf16)x; }
 
-// one wave per (kv head, query)
+// One wave per (kv head, query).  NREG > 0 (scores rounded to bf16, at most 64 * NREG blocks): every block score
+// is packed with its id into one sortable 32-bit key - bf16 bits above, 0xFFFF - id below, so that the larger
+// key is the larger score or, on equal scores, the lower id - and lives in a register; a selection round is a
+// plain unsigned maximum over the wave.  NREG == 0: fp32 scores in LDS, (value, id) compared explicitly.
+template <int NREG>
 __global__ void __launch_bounds__(256)
 cmp_topk_kernel(TopkParams p) {
-  extern __shared__ float bs_all[];  // [4 waves][nblk]
+  extern __shared__ float bs_all[];  // [4 waves][nblk], NREG == 0 only
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int64_t row = (int64_t)blockIdx.x * 4 + wv;
   if (row >= p.n_tokens * p.hkv) return;
@@ -482,7 +486,7 @@ cmp_topk_kernel(TopkParams p) {
   const int n_off = na + ne - 1, pad = na - 1;
   const int bq = qi / p.block_size;
   const float* srow = p.score + ((int64_t)h * p.n_tokens + tok) * p.score_ld;
-  for (int b = lane; b < p.nblk; b += 64) {
+  auto block_score = [&](int b) {
     float acc = 0.f;
     const int c0 = b * ne - pad;
     for (int o = 0; o < n_off; ++o) {
@@ -494,36 +498,54 @@ cmp_topk_kernel(TopkParams p) {
     }
     if (b < p.init_blocks || (bq >= b && bq < b + p.local_blocks)) acc = INFINITY;
     if (p.to_bf16) acc = round_bf16(acc);
-    bs[b] = acc;
     if (p.block_score) p.block_score[((int64_t)h * p.n_tokens + tok) * p.nblk + b] = acc;
-  }
-  __builtin_amdgcn_wave_barrier();
-  // t_out rounds of arg-max by (value desc, id asc); taken entries are marked -1 (scores are >= 0)
-  int my_id = -1;  // lane t keeps the id chosen in round t (t < 64), further rounds spill to LDS-free path
-  for (int t = 0; t < p.t_out; ++t) {
-    float best = -2.f;
-    int best_id = 0x7fffffff;
-    for (int b = lane; b < p.nblk; b += 64) {
-      const float vv = bs[b];
-      if (vv > best) {
-        best = vv;
-        best_id = b;
-      }
-    }
+    return acc;
+  };
+  int my_id = -1;  // lane t keeps the id chosen in round t
+  if (NREG > 0) {
+    uint32_t key[NREG > 0 ? NREG : 1];
 #pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) {
-      const float ov = __shfl_xor(best, o, 64);
-      const int oi = __shfl_xor(best_id, o, 64);
-      if (ov > best || (ov == best && oi < best_id)) {
-        best = ov;
-        best_id = oi;
-      }
+    for (int r = 0; r < NREG; ++r) {
+      const int b = lane + 64 * r;
+      key[r] = b < p.nblk ? ((__float_as_uint(block_score(b)) >> 16 << 16) | (0xFFFFu - (uint32_t)b)) : 0u;
     }
-    if (lane == (t & 63)) {
-      if (t < 64) my_id = best_id;
+    for (int t = 0; t < p.t_out; ++t) {
+      uint32_t best = key[0];
+#pragma unroll
+      for (int r = 1; r < NREG; ++r) best = max(best, key[r]);
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) best = max(best, (uint32_t)__shfl_xor((int)best, o, 64));
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) key[r] = key[r] == best ? 0u : key[r];  // keys are distinct
+      if (lane == t) my_id = 0xFFFF - (int)(best & 0xFFFFu);
     }
-    if (lane == 0) bs[best_id] = -1.f;
+  } else {
+    for (int b = lane; b < p.nblk; b += 64) bs[b] = block_score(b);
     __builtin_amdgcn_wave_barrier();
+    // t_out rounds of arg-max by (value desc, id asc); taken entries are marked -1 (scores are >= 0)
+    for (int t = 0; t < p.t_out; ++t) {
+      float best = -2.f;
+      int best_id = 0x7fffffff;
+      for (int b = lane; b < p.nblk; b += 64) {
+        const float vv = bs[b];
+        if (vv > best) {
+          best = vv;
+          best_id = b;
+        }
+      }
+#pragma unroll
+      for (int o = 32; o >= 1; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(best_id, o, 64);
+        if (ov > best || (ov == best && oi < best_id)) {
+          best = ov;
+          best_id = oi;
+        }
+      }
+      if (lane == t) my_id = best_id;
+      if (lane == 0) bs[best_id] = -1.f;
+      __builtin_amdgcn_wave_barrier();
+    }
   }
   // ascending order by rank counting (ids are distinct), then mask ids above the own block
   const int t_eff = min(p.t_out, 64);
@@ -832,7 +854,12 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   {
     ProfScope ps_("cmp_topk", stream);
     const int64_t rows = total_q * num_kv_heads;
-    cmp_topk_kernel<<<(unsigned)((rows + 3) / 4), 256, (size_t)4 * nblk * 4, stream>>>(tp);
+    const unsigned grid = (unsigned)((rows + 3) / 4);
+    if (scores_to_bf16 && nblk <= 128) cmp_topk_kernel<2><<<grid, 256, 0, stream>>>(tp);
+    else if (scores_to_bf16 && nblk <= 256) cmp_topk_kernel<4><<<grid, 256, 0, stream>>>(tp);
+    else if (scores_to_bf16 && nblk <= 512) cmp_topk_kernel<8><<<grid, 256, 0, stream>>>(tp);
+    else if (scores_to_bf16 && nblk <= 1024) cmp_topk_kernel<16><<<grid, 256, 0, stream>>>(tp);
+    else cmp_topk_kernel<0><<<grid, 256, (size_t)4 * nblk * 4, stream>>>(tp);
   }
   FSA_CHECK_LAUNCH("fsa_cmp_topk select");
   return 0;

@@ -115,3 +115,43 @@ def test_cmp_topk(dev, cu, hq, hkv, d, ks, st, bk, t, dtype):
     same = (idx == want_e2e).all(-1).float().mean().item()
     print(f"  rows identical to the oracle's end-to-end selection: {same:.4f}", flush=True)
     assert same > 0.9
+
+
+# one case per variant of the selection kernel: block scores in 4 / 8 / 16 registers per lane (rounded to bf16),
+# fp32 scores in LDS, more than 1024 blocks in LDS
+TOPK_VARIANTS = [
+    # cu_seqlens, B_K, T, scores_to_bf16
+    ([0, 9000, 21000], 64, 16, True),    # 188 blocks
+    ([0, 15000], 32, 16, True),          # 469 blocks
+    ([0, 40, 20040], 32, 24, True),      # 625 blocks, a sequence shorter than one block
+    ([0, 5000], 64, 16, False),          # fp32 scores
+    ([0, 17000], 16, 16, True),          # 1063 blocks
+]
+
+
+@pytest.mark.parametrize("cu,bk,t,to_bf16", TOPK_VARIANTS)
+def test_cmp_topk_variants(dev, cu, bk, t, to_bf16):
+    print(f"case cu={cu} bk={bk} t={t} to_bf16={to_bf16}", flush=True)
+    hq, hkv, d, ks, st, dtype = 2, 2, 64, 32, 16, torch.bfloat16
+    q, ck, cv, do, cu_k = _make(cu, hq, hkv, d, ks, st, dtype, seed=13)
+    cu_q_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)
+    max_q = max(b - a for a, b in zip(cu[:-1], cu[1:]))
+    max_k = max(b - a for a, b in zip(cu_k[:-1], cu_k[1:]))
+    qd, ckd, cvd = (x.to(dev) for x in (q, ck, cv))
+    o, lse = ops.cmpattn_fwd(qd, ckd, cvd, ks, st, cu_q_t, cu_k_t, max_q)
+    idx, bscore = ops.cmp_topk(qd, ckd, lse, ks, st, bk, t, cu_q_t, cu_k_t, max_q, max_k,
+                               init_blocks=1, local_blocks=2, scores_to_bf16=to_bf16, return_block_score=True)
+    torch.cuda.synchronize()
+    idx, bscore = idx.cpu(), bscore.cpu()
+    want = orc.topk_select_ref(bscore, t, cu, bk, to_bf16=False)   # the scores come back already rounded
+    assert torch.equal(idx, want)
+    if to_bf16:
+        assert torch.equal(bscore.to(torch.bfloat16).float(), bscore)
+    # forced blocks: block 0 and the query's own block are always present
+    n = cu[-1]
+    for a, b in zip(cu[:-1], cu[1:]):
+        own = (torch.arange(b - a) // bk).to(torch.int32)
+        seg = idx[:, a:b]
+        assert (seg[..., 0] == 0).all()
+        assert (seg == own[None, :, None]).any(-1).all()
