@@ -53,7 +53,11 @@ template <int D, int BK> struct SelLds {
   static constexpr int THREADS = TWO_WGS ? 256 : (STAGE8 || !STAGE4) ? 512 : 256;
   static constexpr int NWAVES = THREADS / 64;
   static constexpr bool STAGE_OUT = KV_BYTES + NWAVES * STAGE_BYTES <= 160 * 1024;
-  static constexpr int BYTES = KV_BYTES + (STAGE_OUT ? NWAVES * STAGE_BYTES : 0);
+  // where LDS cannot hold whole-row tiles: a [32][32] slice tile per wave, so that partial rows still leave in
+  // 64-byte pieces, and Q fragments straight from global memory
+  static constexpr int SLS = 32 + 8;
+  static constexpr bool SLICE_OUT = !STAGE_OUT && KV_BYTES + NWAVES * 32 * SLS * 2 <= 160 * 1024;
+  static constexpr int BYTES = KV_BYTES + (STAGE_OUT ? NWAVES * STAGE_BYTES : SLICE_OUT ? NWAVES * 32 * SLS * 2 : 0);
   static constexpr int WG_ROWS = NWAVES * 32;     // rows per pass of the work-group
   static constexpr int MIN_WAVES = (THREADS == 256 && D <= 128 && BK <= 64) ? 2 : 1;  // waves per SIMD the register budget allows
 };
@@ -73,6 +77,8 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   T* Vs = Ks + BK * KS;
   constexpr int OS = SelLds<D, BK>::OS;
   T* Ost = Vs + BK * VS + (threadIdx.x >> 6) * (32 * OS);  // this wave's [32][D] staging tile
+  constexpr int SLS = SelLds<D, BK>::SLS;
+  T* Osl = Vs + BK * VS + (threadIdx.x >> 6) * (32 * SLS);  // or its [32][32] slice tile
 
   const int h = blockIdx.y;
   const int64_t nbp1 = p.max_blocks + 1;
@@ -155,9 +161,11 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       if (sub + SEL_WG_ROWS < row_hi) fetch_q(qst, tok_next, sub + SEL_WG_ROWS);
     } else {
       const int head_ = min(r, row_hi - 1) % p.g;
-      const T* qrow = qbase_row + (int64_t)token * p.q_sn + (int64_t)head_ * p.q_sh + hh * (D / 2);
+      // k-step ks contracts dims [16 ks, 16 ks + 16): the two lanes of a row read 32 contiguous bytes and a
+      // cache line is used up by four consecutive loads
+      const T* qrow = qbase_row + (int64_t)token * p.q_sn + (int64_t)head_ * p.q_sh + hh * 8;
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) qdir[ks] = load16<vec8>(qrow + ks * 8);
+      for (int ks = 0; ks < NKS; ++ks) qdir[ks] = load16<vec8>(qrow + ks * 16);
     }
     f32x16 acc[NA];
 #pragma unroll
@@ -166,7 +174,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
-        vec8 kf = load16<vec8>(&Ks[(a * 32 + col) * KS + hh * (D / 2) + ks * 8]);
+        vec8 kf = load16<vec8>(&Ks[(a * 32 + col) * KS + (STAGED ? hh * (D / 2) + ks * 8 : ks * 16 + hh * 8)]);
         vec8 qf = STAGED ? load16<vec8>(&Ost[col * OS + hh * (D / 2) + ks * 8]) : qdir[STAGED ? 0 : ks];
         acc[a] = Elem<T>::mfma32(kf, qf, acc[a]);
       }
@@ -217,7 +225,18 @@ selattn_fwd_main_kernel(SelFwdParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) x[e] = (T)(oacc[4 * qd + e] * inv_l);
         if (SelLds<D, BK>::STAGE_OUT) store8(&Ost[col * OS + dt * 32 + 8 * qd + 4 * hh], x);
+        else if (SelLds<D, BK>::SLICE_OUT) store8(&Osl[col * SLS + 8 * qd + 4 * hh], x);
         else if (valid) store8(opart + prow * D + dt * 32 + 8 * qd + 4 * hh, x);  // LDS too small: direct
+      }
+      if (SelLds<D, BK>::SLICE_OUT) {  // the 32 dims of this accumulator: 4 lanes per row, 16 rows per store
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int row = (lane >> 2) + 16 * j;
+          vec8 y = load16<vec8>(&Osl[row * SLS + (lane & 3) * 8]);
+          if (sub + row < row_hi) store16(opart + (prow0 + sub + row) * D + dt * 32 + (lane & 3) * 8, y);
+        }
+        __builtin_amdgcn_wave_barrier();
       }
     }
     __builtin_amdgcn_wave_barrier();
