@@ -219,6 +219,25 @@ starts_kernel(const uint32_t* __restrict__ keys, int64_t n_items, int64_t max_bl
   if (gb < max_blocks) counts[h * max_blocks + gb] = lower((uint32_t)gb + 1) - s0;
 }
 
+// out[h, token, t * factor + j] = id of sub-block j of the selected block t, -1 if it lies after the query
+__global__ void __launch_bounds__(256)
+split_blocks_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
+                    const int32_t* __restrict__ cu_seqlens, int batch, int64_t n_out, int topk, int factor,
+                    int sub_size, int32_t* __restrict__ out) {
+  const int h = blockIdx.y;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n_out) return;
+  const int per = topk * factor;
+  const int token = (int)(idx / per);
+  const int r = (int)(idx - (int64_t)token * per);
+  const int t = r / factor, j = r - t * factor;
+  const int b = topk_idx[h * stride_h + (int64_t)token * stride_n + t];
+  const int s = upper_seg(cu_seqlens, batch, token);
+  const int qpos = token - cu_seqlens[s];
+  const int64_t sb = (int64_t)b * factor + j;
+  out[h * n_out + idx] = (b >= 0 && sb * sub_size <= qpos) ? (int32_t)sb : -1;
+}
+
 __global__ void __launch_bounds__(SCAN_THREADS)
 tiles_kernel(const int32_t* __restrict__ counts, int64_t max_blocks, int group_size, int rows_per_tile,
              int32_t* __restrict__ tile_prefix) {
@@ -321,6 +340,24 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
   dim3 g_blocks((unsigned)((max_blocks + 1 + 255) / 256), num_kv_heads);
   starts_kernel<<<g_blocks, 256, 0, stream>>>(keys[cur], n_items, max_blocks, starts, counts);
   FSA_CHECK_LAUNCH("fsa_build_index");
+  return 0;
+}
+
+extern "C" int fsa_split_topk_blocks(const int32_t* topk_idx, int64_t topk_stride_h, int64_t topk_stride_n,
+                                     const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                                     int32_t num_kv_heads, int32_t topk, int32_t block_size, int32_t factor,
+                                     int32_t* out, void* stream_) {
+  FSA_CHECK_ARG(topk_idx && cu_seqlens && out, "fsa_split_topk_blocks: null pointer");
+  FSA_CHECK_ARG(batch >= 1 && total_tokens >= 1 && num_kv_heads >= 1 && topk >= 1,
+                "fsa_split_topk_blocks: batch, total_tokens, num_kv_heads and topk must be positive");
+  FSA_CHECK_ARG(factor >= 1 && block_size >= factor && block_size % factor == 0,
+                "fsa_split_topk_blocks: factor must divide block_size");
+  const int64_t n_out = total_tokens * topk * factor;
+  FSA_CHECK_ARG(n_out < ((int64_t)1 << 31), "fsa_split_topk_blocks: total_tokens*topk*factor must be < 2^31");
+  dim3 grid((unsigned)((n_out + 255) / 256), num_kv_heads);
+  split_blocks_kernel<<<grid, 256, 0, (hipStream_t)stream_>>>(topk_idx, topk_stride_h, topk_stride_n, cu_seqlens,
+                                                             batch, n_out, topk, factor, block_size / factor, out);
+  FSA_CHECK_LAUNCH("fsa_split_topk_blocks");
   return 0;
 }
 

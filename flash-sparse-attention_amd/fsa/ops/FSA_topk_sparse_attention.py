@@ -27,15 +27,16 @@ class PermuteResults(list):
     synchronises); the backward only uses `.index`.
     """
 
-    def __init__(self, index: _ops.SelIndex):
+    def __init__(self, index: _ops.SelIndex, ref_args=None):
         super().__init__()
-        self.index = index
+        self.index = index          # what the kernels use
+        self._ref_args = ref_args   # (topk_idx, cu_seqlens, block_size) when the caller's block size differs
         self._built = False
 
     def _build(self):
         if self._built:
             return
-        ix = self.index
+        ix = self.index if self._ref_args is None else _ops.build_index(*self._ref_args)
         cu = ix.cu_seqlens.cpu().tolist()
         cub = ix.cu_blocks.cpu().tolist()
         for s in range(ix.batch):
@@ -73,6 +74,15 @@ class PermuteResults(list):
         return super().__iter__()
 
 
+def _build_kernel_index(topk_idx, cu_seqlens, block_size):
+    """Index the kernels run on.  Blocks of 256 keys are handled as pairs of 128-key blocks (the same key set
+    for every query); the dicts of `PermuteResults` are still built for the caller's block size."""
+    if block_size == 256:
+        split = _ops.split_topk_blocks(topk_idx, cu_seqlens, 256, 2)
+        return _ops.build_index(split, cu_seqlens, 128), (topk_idx, cu_seqlens, 256)
+    return _ops.build_index(topk_idx, cu_seqlens, block_size), None
+
+
 def _topk_sparse_attention_fwd_opt(
     q: torch.Tensor,  # [total_len, num_q_heads, head_dim]
     k: torch.Tensor,  # [total_len, num_kv_heads, head_dim]
@@ -92,11 +102,9 @@ def _topk_sparse_attention_fwd_opt(
     assert block_size in _BLOCK_SIZES
     assert q.shape[1] % k.shape[1] == 0
     assert causal, "selected attention is causal"
-    if block_size == 256:
-        raise NotImplementedError("block_size 256 is not built into the gfx950 kernels (32, 64, 128 are)")
-    index = _ops.build_index(topk_idx, cu_seqlens_q, block_size)
+    index, ref_args = _build_kernel_index(topk_idx, cu_seqlens_q, block_size)
     o, lse = _ops.selattn_fwd(q, k, v, index, sm_scale)
-    return o, lse, PermuteResults(index)
+    return o, lse, PermuteResults(index, ref_args)
 
 
 def _topk_sparse_attention_bwd_opt(
@@ -119,7 +127,7 @@ def _topk_sparse_attention_bwd_opt(
     assert block_size in _BLOCK_SIZES
     index = getattr(permute_results, "index", None)
     if index is None:
-        index = _ops.build_index(topk_idx, cu_seqlens_q, block_size)
+        index, _ = _build_kernel_index(topk_idx, cu_seqlens_q, block_size)
     return _ops.selattn_bwd(q, k, v, o, do, lse, index, sm_scale)
 
 

@@ -25,6 +25,7 @@ SIGNATURES = {
     "fsa_index_workspace_bytes": (sz, [i64, i32, i32, i64]),
     "fsa_build_index": (C.c_int, [vp, i64, i64, vp, i32, i64, i32, i32, i32, i64,
                                   vp, vp, vp, vp, vp, vp, sz, vp]),
+    "fsa_split_topk_blocks": (C.c_int, [vp, i64, i64, vp, i32, i64, i32, i32, i32, i32, vp, vp]),
     "fsa_build_tiles": (C.c_int, [vp, i32, i64, i32, i32, vp, vp]),
     "fsa_max_tiles": (i64, [i64, i32, i32, i32, i64]),
     "fsa_selattn_fwd_workspace_bytes": (sz, [i64, i32, i32, i32, i32, i64]),

@@ -73,6 +73,22 @@ def build_index(topk_idx: torch.Tensor, cu_seqlens: torch.Tensor, block_size: in
                     sel_tokens, slot_of)
 
 
+def split_topk_blocks(topk_idx: torch.Tensor, cu_seqlens: torch.Tensor, block_size: int, factor: int) -> torch.Tensor:
+    """topk_idx over blocks of `block_size` keys -> [Hkv, N, T*factor] over blocks of block_size // factor keys
+    (sub-blocks that start after the query become -1); the selected key set of every query is unchanged."""
+    _require_cuda(topk_idx, cu_seqlens)
+    assert topk_idx.dtype == torch.int32 and cu_seqlens.dtype == torch.int32
+    assert topk_idx.dim() == 3 and topk_idx.stride(2) == 1
+    lib = _lib.load()
+    hkv, n, t = topk_idx.shape
+    out = torch.empty((hkv, n, t * factor), dtype=torch.int32, device=topk_idx.device)
+    rc = lib.fsa_split_topk_blocks(_ptr(topk_idx), topk_idx.stride(0), topk_idx.stride(1), _ptr(cu_seqlens),
+                                   cu_seqlens.numel() - 1, n, hkv, t, block_size, factor, _ptr(out),
+                                   _stream(topk_idx.device))
+    _lib.check(rc, "fsa_split_topk_blocks")
+    return out
+
+
 def _check_qkv(q, k, v):
     _require_cuda(q, k, v)
     assert q.dtype in _DTYPE, "q must be bf16 or fp16"

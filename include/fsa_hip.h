@@ -77,6 +77,20 @@ int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, int64_t topk
                     int32_t* cu_blocks, int32_t* counts, int32_t* starts, int32_t* sel_tokens,
                     int32_t* slot_of, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Block lists over blocks of `block_size` keys rewritten as lists over blocks
+ * of block_size / factor keys: entry (t, j) of the output is
+ * topk_idx[t] * factor + j when that sub-block starts at or before the query's
+ * position in its sequence, otherwise -1; out is contiguous
+ * [Hkv, N, T * factor].  Attention over the selected blocks is attention over
+ * the union of their keys, so the result is the same operator at a block size
+ * the kernels are built for: this is how block_size 256, which the reference
+ * accepts (fsa/ops/FSA_topk_sparse_attention.py:926), runs on the 128-key
+ * kernels.  No counterpart in the reference. */
+int fsa_split_topk_blocks(const int32_t* topk_idx, int64_t topk_stride_h, int64_t topk_stride_n,
+                          const int32_t* cu_seqlens, int32_t batch, int64_t total_tokens,
+                          int32_t num_kv_heads, int32_t topk, int32_t block_size, int32_t factor,
+                          int32_t* out, void* stream);
+
 /* Work list for the block-major kernels: tile_prefix[h, gb] = number of
  * row tiles of blocks < gb, a row tile being `rows_per_tile` gathered
  * (query, head-in-group) rows of one block.  tile_prefix is [Hkv, max_blocks+1].
