@@ -10,6 +10,8 @@
 #pragma once
 #include "fsa_common.h"
 
+#include <type_traits>
+
 namespace fsa {
 
 struct SelBwdParams {
@@ -173,15 +175,19 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   constexpr bool KLDS = FUSE_DQ && C::K_FROM_LDS;
   vec8 kf[KLDS ? 1 : NS], vf[NS];
   {
-    const T* krow = reinterpret_cast<const T*>(p.k) + (int64_t)ktok * p.k_sn + (int64_t)h * p.k_sh + 8 * kg;
-    const T* vrow = reinterpret_cast<const T*>(p.v) + (int64_t)ktok * p.v_sn + (int64_t)h * p.v_sh + 8 * kg;
+    // Contraction index of the S / dP products: k-step s_ covers dims [32 s_, 32 s_ + 32); the lane of key
+    // group kg holds dims 4 kg .. 4 kg + 3 and 16 + 4 kg .. 16 + 4 kg + 3 of it.  Both halves are 8-byte
+    // pieces, so the matching Q / dO fragments come from LDS with 8-byte reads in which the four key groups
+    // read 32 contiguous bytes of a row (full LDS rate; a 16-byte read per lane runs at half of it).
+    const T* krow = reinterpret_cast<const T*>(p.k) + (int64_t)ktok * p.k_sn + (int64_t)h * p.k_sh + 4 * kg;
+    const T* vrow = reinterpret_cast<const T*>(p.v) + (int64_t)ktok * p.v_sn + (int64_t)h * p.v_sh + 4 * kg;
 #pragma unroll
     for (int s_ = 0; s_ < NS; ++s_) {
       if (!KLDS) kf[s_] = zero8<T>();
       vf[s_] = zero8<T>();
       if (key_ok) {
-        if (!KLDS) kf[s_] = load16<vec8>(krow + 32 * s_);
-        vf[s_] = load16<vec8>(vrow + 32 * s_);
+        if (!KLDS) kf[s_] = load8x2<T>(krow + 32 * s_);
+        vf[s_] = load8x2<T>(vrow + 32 * s_);
       }
     }
   }
@@ -273,8 +279,9 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     }
 
   // lane addresses: A operand rows (natural) and transposing reads
-  const int a_off = l16 * QS + 8 * kg;                            // + rt*16*QS + 32*s
+  const int a_off = l16 * QS + 4 * kg;                            // + rt*16*QS + 32*s (+ 16 for the second half)
   const int tr_off = (4 * kg + (l16 >> 2)) * QS + 4 * (l16 & 3);  // + 32*u*QS + 16*dtile
+
 
   fetch_tokens(row_lo);
   fetch(row_lo);
@@ -289,27 +296,97 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     }
 
     vec4 pk[NRT], dsk[NRT];
+    // Q / dO fragments of row tile rt: [Q lo s_ | Q hi s_ | dO lo s_ | dO hi s_], issued one row tile ahead
+    constexpr bool RAW = !KLDS && NS <= 4;
+    constexpr int NF = RAW ? 4 * NS : 1;
+    u32x2 fr[2][NF];
+    // statistics of the lane's four rows of the tile: [lse 0-1 | lse 2-3 | delta 0-1 | delta 2-3 | limit 0-1 |
+    // limit 2-3 (| lower limit 0-1 | 2-3 in window mode)]
+    constexpr int NST = RAW ? (MODE == KV_MODE_WINDOW ? 8 : 6) : 1;
+    u32x2 st[2][NST];
+    const uint32_t a_addr = lds_addr(Qs + a_off);
+    const uint32_t s_addr = lds_addr(lse_s + 4 * kg);
+    constexpr int O_BYTES = C::KV_R * QS * 2;  // Os - Qs
+    constexpr int STAT_BYTES = C::KV_R * 4;    // del_s - lse_s = lim_s - del_s = llo_s - lim_s
+    auto issue = [&](auto rt_c, u32x2 (&dst)[NF]) {
+      constexpr int rt = decltype(rt_c)::value;
+      if constexpr (RAW) {
+        constexpr int RB = rt * 16 * QS * 2;
+        u32x2 (&sd)[NST] = st[rt & 1];
 #pragma unroll
-    for (int rt = 0; rt < NRT; ++rt) {
-      f32x4 sacc = {0.f, 0.f, 0.f, 0.f}, dpacc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s_ = 0; s_ < NS; ++s_) {
-        vec8 qa = load16<vec8>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
-        sacc = Elem<T>::mfma16(qa, KLDS ? load16<vec8>(&Kl[key * C::KS + 32 * s_ + 8 * kg]) : kf[KLDS ? 0 : s_], sacc);
-        vec8 da = load16<vec8>(&Os[rt * 16 * QS + a_off + 32 * s_]);
-        dpacc = Elem<T>::mfma16(da, vf[s_], dpacc);
-        if (C::TIGHT_REGS && (s_ & 1) == 1) asm volatile("" ::: "memory");
+        for (int a_ = 0; a_ < NST / 2; ++a_) {  // unrolled: the offsets below are constants
+          if (a_ == 0) { sd[0] = lds_read8_raw<rt * 64>(s_addr); sd[1] = lds_read8_raw<rt * 64 + 8>(s_addr); }
+          if (a_ == 1) { sd[2] = lds_read8_raw<STAT_BYTES + rt * 64>(s_addr); sd[3] = lds_read8_raw<STAT_BYTES + rt * 64 + 8>(s_addr); }
+          if (a_ == 2) { sd[4] = lds_read8_raw<2 * STAT_BYTES + rt * 64>(s_addr); sd[5] = lds_read8_raw<2 * STAT_BYTES + rt * 64 + 8>(s_addr); }
+          if (a_ == 3) { sd[NST - 2] = lds_read8_raw<3 * STAT_BYTES + rt * 64>(s_addr); sd[NST - 1] = lds_read8_raw<3 * STAT_BYTES + rt * 64 + 8>(s_addr); }
+        }
+        dst[0] = lds_read8_raw<RB>(a_addr);
+        dst[NS] = lds_read8_raw<RB + 32>(a_addr);
+        dst[2 * NS] = lds_read8_raw<O_BYTES + RB>(a_addr);
+        dst[3 * NS] = lds_read8_raw<O_BYTES + RB + 32>(a_addr);
+        if constexpr (NS > 1) {
+          dst[1] = lds_read8_raw<RB + 64>(a_addr);
+          dst[NS + 1] = lds_read8_raw<RB + 96>(a_addr);
+          dst[2 * NS + 1] = lds_read8_raw<O_BYTES + RB + 64>(a_addr);
+          dst[3 * NS + 1] = lds_read8_raw<O_BYTES + RB + 96>(a_addr);
+        }
+        if constexpr (NS > 2) {
+          dst[2] = lds_read8_raw<RB + 128>(a_addr);
+          dst[NS + 2] = lds_read8_raw<RB + 160>(a_addr);
+          dst[2 * NS + 2] = lds_read8_raw<O_BYTES + RB + 128>(a_addr);
+          dst[3 * NS + 2] = lds_read8_raw<O_BYTES + RB + 160>(a_addr);
+          dst[3] = lds_read8_raw<RB + 192>(a_addr);
+          dst[NS + 3] = lds_read8_raw<RB + 224>(a_addr);
+          dst[2 * NS + 3] = lds_read8_raw<O_BYTES + RB + 192>(a_addr);
+          dst[3 * NS + 3] = lds_read8_raw<O_BYTES + RB + 224>(a_addr);
+        }
       }
-      const float4 lse4 = *reinterpret_cast<const float4*>(&lse_s[rt * 16 + 4 * kg]);
-      const float4 del4 = *reinterpret_cast<const float4*>(&del_s[rt * 16 + 4 * kg]);
-      const int4 lim4 = *reinterpret_cast<const int4*>(&lim_s[rt * 16 + 4 * kg]);
-      const float lse_r[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
-      const float del_r[4] = {del4.x, del4.y, del4.z, del4.w};
-      const int lim_r[4] = {lim4.x, lim4.y, lim4.z, lim4.w};
-      int llo_r[4] = {0, 0, 0, 0};
-      if (MODE == KV_MODE_WINDOW) {
-        const int4 llo4 = *reinterpret_cast<const int4*>(&llo_s[rt * 16 + 4 * kg]);
-        llo_r[0] = llo4.x; llo_r[1] = llo4.y; llo_r[2] = llo4.z; llo_r[3] = llo4.w;
+    };
+    auto s_phase = [&](auto rt_c) {
+      constexpr int rt = decltype(rt_c)::value;
+      f32x4 sacc = {0.f, 0.f, 0.f, 0.f}, dpacc = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (RAW) {
+        u32x2 (&cur)[NF] = fr[rt & 1];
+        lds_wait<NF>(cur);
+        lds_wait<NST>(st[rt & 1]);
+        if constexpr (rt + 1 < NRT) issue(std::integral_constant<int, rt + 1>{}, fr[(rt + 1) & 1]);
+#pragma unroll
+        for (int s_ = 0; s_ < NS; ++s_) {
+          sacc = Elem<T>::mfma16(frag8<T>(cur[s_], cur[NS + s_]), kf[KLDS ? 0 : s_], sacc);
+          dpacc = Elem<T>::mfma16(frag8<T>(cur[2 * NS + s_], cur[3 * NS + s_]), vf[s_], dpacc);
+        }
+      } else {
+#pragma unroll
+        for (int s_ = 0; s_ < NS; ++s_) {
+          vec8 qa = load8x2<T>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
+          sacc = Elem<T>::mfma16(qa, KLDS ? load8x2<T>(&Kl[key * C::KS + 32 * s_ + 4 * kg]) : kf[KLDS ? 0 : s_], sacc);
+          vec8 da = load8x2<T>(&Os[rt * 16 * QS + a_off + 32 * s_]);
+          dpacc = Elem<T>::mfma16(da, vf[s_], dpacc);
+          if (C::TIGHT_REGS && (s_ & 1) == 1) asm volatile("" ::: "memory");
+        }
+      }
+      float lse_r[4], del_r[4];
+      int lim_r[4], llo_r[4] = {0, 0, 0, 0};
+      if constexpr (RAW) {
+        u32x2 (&sd)[NST] = st[rt & 1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          lse_r[i] = __uint_as_float(sd[i >> 1][i & 1]);
+          del_r[i] = __uint_as_float(sd[2 + (i >> 1)][i & 1]);
+          lim_r[i] = (int)sd[4 + (i >> 1)][i & 1];
+          if (MODE == KV_MODE_WINDOW) llo_r[i] = (int)sd[NST - 2 + (i >> 1)][i & 1];
+        }
+      } else {
+        const float4 lse4 = *reinterpret_cast<const float4*>(&lse_s[rt * 16 + 4 * kg]);
+        const float4 del4 = *reinterpret_cast<const float4*>(&del_s[rt * 16 + 4 * kg]);
+        const int4 lim4 = *reinterpret_cast<const int4*>(&lim_s[rt * 16 + 4 * kg]);
+        lse_r[0] = lse4.x; lse_r[1] = lse4.y; lse_r[2] = lse4.z; lse_r[3] = lse4.w;
+        del_r[0] = del4.x; del_r[1] = del4.y; del_r[2] = del4.z; del_r[3] = del4.w;
+        lim_r[0] = lim4.x; lim_r[1] = lim4.y; lim_r[2] = lim4.z; lim_r[3] = lim4.w;
+        if (MODE == KV_MODE_WINDOW) {
+          const int4 llo4 = *reinterpret_cast<const int4*>(&llo_s[rt * 16 + 4 * kg]);
+          llo_r[0] = llo4.x; llo_r[1] = llo4.y; llo_r[2] = llo4.z; llo_r[3] = llo4.w;
+        }
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -319,7 +396,15 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         pk[rt][i] = (T)pv;
         dsk[rt][i] = (T)ds;
       }
+    };
+    issue(std::integral_constant<int, 0>{}, fr[0]);
+    s_phase(std::integral_constant<int, 0>{});
+    s_phase(std::integral_constant<int, 1>{});
+    if constexpr (NRT > 2) {
+      s_phase(std::integral_constant<int, 2>{});
+      s_phase(std::integral_constant<int, 3>{});
     }
+    static_assert(NRT == 2 || NRT == 4, "row tiles per pass");
     if (FUSE_DQ) {
       // dS^T[key][row] for the whole tile: every lane owns 4 consecutive rows of its key
 #pragma unroll

@@ -62,6 +62,49 @@ template <typename V> __device__ __forceinline__ void store8(void* p, V v) {
   *reinterpret_cast<uint2*>(p) = __builtin_bit_cast(uint2, v);
 }
 
+// elements p[0..3] and p[16..19] as one 8-element fragment (two 8-byte moves)
+template <typename T> __device__ __forceinline__ typename Elem<T>::vec8 load8x2(const T* p) {
+  typename Elem<T>::vec4 lo = load8<typename Elem<T>::vec4>(p);
+  typename Elem<T>::vec4 hi = load8<typename Elem<T>::vec4>(p + 16);
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// ---- hand-issued 8-byte LDS reads --------------------------------------------------------------
+// An LDS instruction that returns 16 bytes per lane (ds_read_b128, ds_read2_b64) delivers 64 bytes per clock
+// on gfx950, an 8-byte one (ds_read_b64) 128.  The compiler fuses neighbouring 8-byte reads into the 16-byte
+// forms, so the reads that should stay separate are issued by hand.  The compiler does not know that their
+// results are still in flight: lds_wait() has to be placed between such reads and the first use of their
+// results, with every result passed through it.
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint32_t lds_addr(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+template <int OFFSET_BYTES> __device__ __forceinline__ u32x2 lds_read8_raw(uint32_t addr) {
+  static_assert(OFFSET_BYTES >= 0 && OFFSET_BYTES < 65536, "ds offset field");
+  u32x2 r;
+  asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFFSET_BYTES));
+  return r;
+}
+template <int N> __device__ __forceinline__ void lds_wait(u32x2 (&r)[N]);
+template <> __device__ __forceinline__ void lds_wait<6>(u32x2 (&r)[6]) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]));
+}
+template <> __device__ __forceinline__ void lds_wait<8>(u32x2 (&r)[8]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
+}
+template <> __device__ __forceinline__ void lds_wait<16>(u32x2 (&r)[16]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]),
+                 "+v"(r[8]), "+v"(r[9]), "+v"(r[10]), "+v"(r[11]), "+v"(r[12]), "+v"(r[13]), "+v"(r[14]),
+                 "+v"(r[15]));
+}
+template <typename T> __device__ __forceinline__ typename Elem<T>::vec8 frag8(u32x2 lo, u32x2 hi) {
+  u32x4 x = {lo[0], lo[1], hi[0], hi[1]};
+  return __builtin_bit_cast(typename Elem<T>::vec8, x);
+}
+
 template <typename T> __device__ __forceinline__ typename Elem<T>::vec8 zero8() {
   uint4 z = make_uint4(0, 0, 0, 0);
   return __builtin_bit_cast(typename Elem<T>::vec8, z);
