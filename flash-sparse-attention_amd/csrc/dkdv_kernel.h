@@ -33,6 +33,7 @@ struct SelBwdParams {
   int64_t cap;
   int64_t n_tokens;
   int g;
+  int g_shift;  // log2 g, or -1 if g is not a power of two
   float scale;
   float scale_log2;
   void* dq_part;     // [Hkv, cap, g, D] lane-native order
@@ -204,8 +205,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   const int32_t* toks = MODE == KV_MODE_SELECTED ? p.sel_tokens + (int64_t)h * p.cap + start : nullptr;
   // row r of the block -> global query row
   auto row_token = [&](int r) {
-    if (MODE == KV_MODE_SELECTED) return (int)toks[r / p.g];
-    return blk.seq_start + blk.q_first + r / p.g;
+    if (MODE == KV_MODE_SELECTED) return (int)toks[div_group(r, p.g, p.g_shift)];
+    return blk.seq_start + blk.q_first + div_group(r, p.g, p.g_shift);
   };
   const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)h * p.g * p.q_sh;
   const T* dobase = reinterpret_cast<const T*>(p.d_o) + (int64_t)h * p.g * p.do_sh;
@@ -231,7 +232,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       qst[j] = zero8<T>();
       dost[j] = zero8<T>();
       if (r < row_hi) {
-        const int trank = r / p.g, head = r - trank * p.g;
+        const int trank = div_group(r, p.g, p.g_shift), head = r - trank * p.g;
         const int token = tok_pf[j];
         qst[j] = load16<vec8>(qbase + (int64_t)token * p.q_sn + (int64_t)head * p.q_sh + ld_col * 8);
         dost[j] = load16<vec8>(dobase + (int64_t)token * p.do_sn + (int64_t)head * p.do_sh + ld_col * 8);
@@ -244,7 +245,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       lim_st = -1;
       llo_st = 0;
       if (r < row_hi) {
-        const int trank = r / p.g, head = r - trank * p.g;
+        const int trank = div_group(r, p.g, p.g_shift), head = r - trank * p.g;
         const int token = tok_stat;
         const int64_t stat = (int64_t)(h * p.g + head) * p.n_tokens + token;
         lse_st = p.lse[stat];

@@ -138,6 +138,17 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// r / g for a row index r >= 0 and a GQA group of g heads: a shift where g is a power of two (g_shift =
+// log2 g), the division otherwise (g_shift < 0).  The general division costs some forty instructions and sits in
+// the address computation of every gathered row.
+__device__ __forceinline__ int div_group(int r, int g, int g_shift) { return g_shift >= 0 ? (r >> g_shift) : r / g; }
+static inline int group_shift(int g) {
+  if (g <= 0 || (g & (g - 1)) != 0) return -1;
+  int s = 0;
+  while ((1 << s) < g) ++s;
+  return s;
+}
+
 // largest i in [0, n) with a[i] <= x, for ascending a[0..n) with a[0] <= x
 __device__ __forceinline__ int upper_seg(const int32_t* __restrict__ a, int n, int x) {
   int lo = 0, hi = n;  // invariant a[lo] <= x, a[hi] > x (virtual)

@@ -114,7 +114,7 @@ selattn_bwd_dq_kernel(SelBwdParams p) {
     const int r = sub + col;
     const bool valid = r < row_hi;
     const int rr = valid ? r : row_hi - 1;
-    const int trank = rr / p.g;
+    const int trank = div_group(rr, p.g, p.g_shift);
     const int head = rr - trank * p.g;
     const int token = toks[trank];
     const T* qrow = qbase + (int64_t)token * p.q_sn + (int64_t)head * p.q_sh;
@@ -415,7 +415,7 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   p.v_sn = v_stride_n; p.v_sh = v_stride_h; p.do_sn = do_stride_n; p.do_sh = do_stride_h;
   p.cu_seqlens = cu_seqlens; p.cu_blocks = cu_blocks; p.counts = counts; p.starts = starts;
   p.sel_tokens = sel_tokens;
-  p.batch = batch; p.max_blocks = max_blocks; p.cap = cap; p.n_tokens = total_tokens; p.g = g;
+  p.batch = batch; p.max_blocks = max_blocks; p.cap = cap; p.n_tokens = total_tokens; p.g = g; p.g_shift = group_shift(g);
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * LOG2E;
   p.dq_part = wsp + ws.off_dqpart;
   p.dkdv_part = (float*)(wsp + ws.off_kvpart);

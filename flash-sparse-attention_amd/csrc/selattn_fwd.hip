@@ -32,6 +32,7 @@ struct SelFwdParams {
   int64_t max_blocks;
   int64_t cap;  // N * T: capacity of the per-head pair list
   int g;
+  int g_shift;  // log2 g, or -1 if g is not a power of two
   float scale_log2;
   void* o_part;
   float* lse_part;
@@ -134,7 +135,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   const int srow = lane / CPR, schunk = lane % CPR;
   auto row_token = [&](int sub_) {  // token id of row (sub_ + col), kept by lane col
     const int r_ = min(sub_ + col, row_hi - 1);
-    return toks[r_ / p.g];
+    return toks[div_group(r_, p.g, p.g_shift)];
   };
   auto fetch_q = [&](vec8 (&dst)[NLD], int tok_lane, int sub_) {
 #pragma unroll
@@ -142,7 +143,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       const int row = srow + RPI * j;
       const int tok_ = __shfl(tok_lane, row, 64);
       const int r_ = min(sub_ + row, row_hi - 1);
-      const int head_ = r_ % p.g;
+      const int head_ = r_ - div_group(r_, p.g, p.g_shift) * p.g;
       dst[j] = load16<vec8>(qbase_row + (int64_t)tok_ * p.q_sn + (int64_t)head_ * p.q_sh + schunk * 8);
     }
   };
@@ -160,7 +161,8 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       __builtin_amdgcn_wave_barrier();
       if (sub + SEL_WG_ROWS < row_hi) fetch_q(qst, tok_next, sub + SEL_WG_ROWS);
     } else {
-      const int head_ = min(r, row_hi - 1) % p.g;
+      const int rc_ = min(r, row_hi - 1);
+      const int head_ = rc_ - div_group(rc_, p.g, p.g_shift) * p.g;
       // k-step ks contracts dims [16 ks, 16 ks + 16): the two lanes of a row read 32 contiguous bytes and a
       // cache line is used up by four consecutive loads
       const T* qrow = qbase_row + (int64_t)token * p.q_sn + (int64_t)head_ * p.q_sh + hh * 8;
@@ -456,6 +458,7 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
   p.cu_seqlens = cu_seqlens; p.cu_blocks = cu_blocks; p.counts = counts; p.starts = starts;
   p.sel_tokens = sel_tokens; p.tile_prefix = tile_prefix;
   p.batch = batch; p.max_blocks = max_blocks; p.cap = total_tokens * topk; p.g = g;
+  p.g_shift = group_shift(g);
   p.scale_log2 = softmax_scale * LOG2E;
   p.o_part = wsp + ws.off_opart;
   p.lse_part = (float*)(wsp + ws.off_lse);
