@@ -8,6 +8,8 @@
 // N*T; nothing of size nblk*N is ever materialised.
 #include "fsa_common.h"
 
+#include <stdlib.h>
+
 namespace fsa {
 
 constexpr int RS_THREADS = 256;
@@ -219,6 +221,173 @@ starts_kernel(const uint32_t* __restrict__ keys, int64_t n_items, int64_t max_bl
   if (gb < max_blocks) counts[h * max_blocks + gb] = lower((uint32_t)gb + 1) - s0;
 }
 
+// ------------------------------------------------------------------------------------------------
+// Counting path (a few thousand blocks at most): one pass that counts, per tile of consecutive queries,
+// the entries of every block, a scan of those counts over the tiles, and one pass that places every entry:
+// position = start of its block + entries of the block in earlier tiles + earlier entries of the block inside
+// the tile.  Entries are visited in (query, slot) order, so every block's list is ascending in the query id.
+// Padding entries form one extra "block" (id max_blocks) behind all others: the -1 tail of sel_tokens.
+constexpr int CT_THREADS = 256;
+constexpr int CT_WAVES = CT_THREADS / WAVE;
+constexpr int CT_ITEMS = 4096;                       // entries per tile (a whole number of queries)
+constexpr int CT_ROUNDS = CT_ITEMS / CT_THREADS;     // entries per thread
+constexpr int CT_MAX_BUCKETS = 4096;                 // max_blocks + 1 must not exceed this (LDS: 16 B per bucket)
+
+__device__ __forceinline__ int item_bucket(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
+                                           const int32_t* __restrict__ cu_seqlens,
+                                           const int32_t* __restrict__ cu_blocks, int batch, int h, int token,
+                                           int t, int sentinel) {
+  const int b = topk_idx[h * stride_h + (int64_t)token * stride_n + t];
+  const int s = upper_seg(cu_seqlens, batch, token);
+  const int b0 = cu_blocks[s], nb = cu_blocks[s + 1] - b0;
+  return (b >= 0 && b < nb) ? b0 + b : sentinel;
+}
+
+// table[h][bucket][tile] = entries of the tile that fall into the bucket
+__global__ void __launch_bounds__(CT_THREADS)
+count_tiles_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
+                   const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ cu_blocks, int batch,
+                   int64_t n_tokens, int topk, int q_per_tile, int ntiles, int nbuckets,
+                   int32_t* __restrict__ table) {
+  extern __shared__ int hist[];
+  const int h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+  for (int b = tid; b < nbuckets; b += CT_THREADS) hist[b] = 0;
+  __syncthreads();
+  const int64_t tok0 = (int64_t)tile * q_per_tile;
+  const int n_q = (int)min((int64_t)q_per_tile, n_tokens - tok0);
+  for (int i = tid; i < n_q * topk; i += CT_THREADS) {
+    const int qi = i / topk, t = i - qi * topk;
+    atomicAdd(&hist[item_bucket(topk_idx, stride_h, stride_n, cu_seqlens, cu_blocks, batch, h, (int)tok0 + qi, t,
+                                nbuckets - 1)], 1);
+  }
+  __syncthreads();
+  for (int b = tid; b < nbuckets; b += CT_THREADS) table[((int64_t)h * nbuckets + b) * ntiles + tile] = hist[b];
+}
+
+// one wave per (head, bucket): exclusive scan of its row of the table over the tiles; the row total is the
+// bucket's entry count
+__global__ void __launch_bounds__(CT_THREADS)
+scan_tiles_kernel(int32_t* __restrict__ table, int ntiles, int nbuckets, int64_t max_blocks,
+                  int32_t* __restrict__ counts, int32_t* __restrict__ bucket_total) {
+  const int h = blockIdx.y, lane = threadIdx.x & (WAVE - 1);
+  const int b = blockIdx.x * CT_WAVES + threadIdx.x / WAVE;
+  if (b >= nbuckets) return;
+  int32_t* row = table + ((int64_t)h * nbuckets + b) * ntiles;
+  int carry = 0;
+  for (int base = 0; base < ntiles; base += WAVE) {
+    const int i = base + lane;
+    const int v = i < ntiles ? row[i] : 0;
+    int inc = v;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+      const int t = __shfl_up(inc, o, WAVE);
+      if (lane >= o) inc += t;
+    }
+    if (i < ntiles) row[i] = carry + inc - v;
+    carry += __shfl(inc, WAVE - 1, WAVE);
+  }
+  if (lane == 0) {
+    bucket_total[h * nbuckets + b] = carry;
+    if (b < max_blocks) counts[h * max_blocks + b] = carry;
+  }
+}
+
+// starts[h][0..max_blocks] = exclusive scan of the bucket totals (the padding bucket starts where the last
+// block ends)
+__global__ void __launch_bounds__(SCAN_THREADS)
+bucket_starts_kernel(const int32_t* __restrict__ bucket_total, int nbuckets, int32_t* __restrict__ starts) {
+  const int h = blockIdx.x;
+  const int32_t* c = bucket_total + h * nbuckets;
+  int32_t* st = starts + h * nbuckets;  // [Hkv, max_blocks + 1] with nbuckets = max_blocks + 1
+  const int per = (nbuckets + SCAN_THREADS - 1) / SCAN_THREADS;
+  const int lo = min(nbuckets, (int)threadIdx.x * per), hi = min(nbuckets, lo + per);
+  int sum = 0;
+  for (int i = lo; i < hi; ++i) sum += c[i];
+  int total;
+  int run = block_exclusive_scan(sum, &total);
+  for (int i = lo; i < hi; ++i) {
+    st[i] = run;
+    run += c[i];
+  }
+}
+
+__global__ void __launch_bounds__(CT_THREADS)
+place_items_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
+                   const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ cu_blocks, int batch,
+                   int64_t n_tokens, int topk, int q_per_tile, int ntiles, int nbuckets, int key_bits,
+                   const int32_t* __restrict__ table, const int32_t* __restrict__ starts,
+                   int32_t* __restrict__ sel_tokens, int32_t* __restrict__ slot_of) {
+  extern __shared__ int cnt[];  // [CT_WAVES][nbuckets]
+  const int h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid & (WAVE - 1), w = tid / WAVE;
+  for (int i = tid; i < CT_WAVES * nbuckets; i += CT_THREADS) cnt[i] = 0;
+  __syncthreads();
+  const int64_t tok0 = (int64_t)tile * q_per_tile;
+  const int n_q = (int)min((int64_t)q_per_tile, n_tokens - tok0);
+  const int n_it = n_q * topk;
+  // wave w owns entries [w * per_wave, (w + 1) * per_wave) of the tile, 64 per round, in order
+  const int per_wave = (q_per_tile * topk + CT_WAVES - 1) / CT_WAVES;
+  const int rounds = (per_wave + WAVE - 1) / WAVE;   // <= CT_ROUNDS (host check)
+  int key[CT_ROUNDS], rank[CT_ROUNDS];
+  const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  int* my_cnt = cnt + w * nbuckets;
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r) {
+    key[r] = -1;
+    rank[r] = 0;
+    if (r < rounds) {  // uniform
+      const int i = w * per_wave + r * WAVE + lane;
+      const bool ok = r * WAVE + lane < per_wave && i < n_it;
+      int kb = 0;
+      if (ok) {
+        const int qi = i / topk, t = i - qi * topk;
+        kb = item_bucket(topk_idx, stride_h, stride_n, cu_seqlens, cu_blocks, batch, h, (int)tok0 + qi, t,
+                         nbuckets - 1);
+        key[r] = kb;
+      }
+      uint64_t peers = __ballot(ok);
+      for (int bit = 0; bit < key_bits; ++bit) {
+        const bool one = (kb >> bit) & 1;
+        const uint64_t bb = __ballot(one);
+        peers &= one ? bb : ~bb;
+      }
+      int old = 0;
+      if (ok) {
+        old = my_cnt[kb];
+        rank[r] = old + __popcll(peers & lt_mask);
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (ok && (peers & lt_mask) == 0) my_cnt[kb] = old + __popcll(peers);
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  __syncthreads();
+  // per bucket: first position of this tile's entries, then the exclusive prefix over the waves
+  for (int b = tid; b < nbuckets; b += CT_THREADS) {
+    int run = starts[h * nbuckets + b] + table[((int64_t)h * nbuckets + b) * ntiles + tile];
+#pragma unroll
+    for (int ww = 0; ww < CT_WAVES; ++ww) {
+      const int c = cnt[ww * nbuckets + b];
+      cnt[ww * nbuckets + b] = run;
+      run += c;
+    }
+  }
+  __syncthreads();
+  const int64_t n_items = n_tokens * topk;
+  int32_t* st = sel_tokens + h * n_items;
+  int32_t* so = slot_of + h * n_items;
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r) {
+    if (r < rounds && key[r] >= 0) {
+      const int i = w * per_wave + r * WAVE + lane;
+      const int pos = my_cnt[key[r]] + rank[r];
+      const bool real = key[r] != nbuckets - 1;
+      st[pos] = real ? (int32_t)(tok0 + i / topk) : -1;
+      so[tok0 * topk + i] = real ? pos : -1;
+    }
+  }
+}
+
 // out[h, token, t * factor + j] = id of sub-block j of the selected block t, -1 if it lies after the query
 __global__ void __launch_bounds__(256)
 split_blocks_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
@@ -278,9 +447,32 @@ static void index_ws_layout(int64_t n_items, int hkv, size_t* off_keys, size_t* 
   *total = *off_totals + align_up((size_t)hkv * 256 * 4, 256);
 }
 
+// The counting path needs max_blocks + 1 buckets in LDS (16 bytes each), at most CT_ROUNDS entries per thread
+// and a [Hkv, buckets, tiles] table of moderate size; everything else takes the radix sort.
+struct CountPlan {
+  bool use;
+  int q_per_tile, ntiles, nbuckets;
+  size_t off_table, off_totals, total;
+};
+static CountPlan count_plan(int64_t total_tokens, int topk, int hkv, int64_t max_blocks) {
+  CountPlan c = {};
+  if (max_blocks + 1 > CT_MAX_BUCKETS || topk > CT_ITEMS / 4) return c;
+  c.q_per_tile = CT_ITEMS / topk;
+  c.ntiles = (int)((total_tokens + c.q_per_tile - 1) / c.q_per_tile);
+  c.nbuckets = (int)max_blocks + 1;
+  const size_t entries = (size_t)hkv * c.nbuckets * c.ntiles;
+  if (entries > ((size_t)1 << 24)) return c;
+  c.use = getenv("FSA_INDEX_RADIX") == nullptr;  // the environment switch forces the general path (for tests)
+  c.off_table = 0;
+  c.off_totals = align_up(entries * 4, 256);
+  c.total = c.off_totals + align_up((size_t)hkv * c.nbuckets * 4, 256);
+  return c;
+}
+
 extern "C" size_t fsa_index_workspace_bytes(int64_t total_tokens, int32_t topk, int32_t num_kv_heads,
                                             int64_t max_blocks) {
-  (void)max_blocks;
+  const CountPlan c = count_plan(total_tokens, topk, num_kv_heads, max_blocks);
+  if (c.use) return c.total;
   size_t ok[2], ov[2], ot, ott, total;
   index_ws_layout(total_tokens * topk, num_kv_heads, ok, ov, &ot, &ott, &total);
   return total;
@@ -302,13 +494,48 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
                 "fsa_build_index: max_blocks=%lld out of range", (long long)max_blocks);
   const int64_t n_items = total_tokens * topk;
   FSA_CHECK_ARG(n_items < ((int64_t)1 << 31), "fsa_build_index: total_tokens*topk must be < 2^31");
-  size_t ok[2], ov[2], ot, ott, total;
-  index_ws_layout(n_items, num_kv_heads, ok, ov, &ot, &ott, &total);
-  if (workspace == nullptr || workspace_bytes < total) {
-    set_error("fsa_build_index: workspace too small (%zu < %zu)", workspace_bytes, total);
+  const size_t need = fsa_index_workspace_bytes(total_tokens, topk, num_kv_heads, max_blocks);
+  if (workspace == nullptr || workspace_bytes < need) {
+    set_error("fsa_build_index: workspace too small (%zu < %zu)", workspace_bytes, need);
     return FSA_ERR_WORKSPACE;
   }
   char* ws = (char*)workspace;
+  ProfScope ps_("index_build", stream);  // the whole pipeline of small kernels as one record
+  cu_blocks_kernel<<<1, 64, 0, stream>>>(cu_seqlens, batch, block_size, cu_blocks);
+
+  const CountPlan c = count_plan(total_tokens, topk, num_kv_heads, max_blocks);
+  if (c.use) {
+    int32_t* table = (int32_t*)(ws + c.off_table);
+    int32_t* totals = (int32_t*)(ws + c.off_totals);
+    int key_bits = 1;
+    while ((1 << key_bits) < c.nbuckets) ++key_bits;
+    dim3 g_tiles(c.ntiles, num_kv_heads);
+    count_tiles_kernel<<<g_tiles, CT_THREADS, (size_t)c.nbuckets * 4, stream>>>(
+        topk_idx, topk_stride_h, topk_stride_n, cu_seqlens, cu_blocks, batch, total_tokens, topk, c.q_per_tile,
+        c.ntiles, c.nbuckets, table);
+    scan_tiles_kernel<<<dim3((c.nbuckets + CT_WAVES - 1) / CT_WAVES, num_kv_heads), CT_THREADS, 0, stream>>>(
+        table, c.ntiles, c.nbuckets, max_blocks, counts, totals);
+    bucket_starts_kernel<<<num_kv_heads, SCAN_THREADS, 0, stream>>>(totals, c.nbuckets, starts);
+    const size_t lds = (size_t)CT_WAVES * c.nbuckets * 4;
+    static bool attr_done = false;
+    if (!attr_done && lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void*)place_items_kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, CT_WAVES * CT_MAX_BUCKETS * 4);
+      if (e != hipSuccess) {
+        set_error("hipFuncSetAttribute(place_items_kernel): %s", hipGetErrorString(e));
+        return (int)e;
+      }
+      attr_done = true;
+    }
+    place_items_kernel<<<g_tiles, CT_THREADS, lds, stream>>>(
+        topk_idx, topk_stride_h, topk_stride_n, cu_seqlens, cu_blocks, batch, total_tokens, topk, c.q_per_tile,
+        c.ntiles, c.nbuckets, key_bits, table, starts, sel_tokens, slot_of);
+    FSA_CHECK_LAUNCH("fsa_build_index");
+    return 0;
+  }
+
+  size_t ok[2], ov[2], ot, ott, total;
+  index_ws_layout(n_items, num_kv_heads, ok, ov, &ot, &ott, &total);
   uint32_t* keys[2] = {(uint32_t*)(ws + ok[0]), (uint32_t*)(ws + ok[1])};
   uint32_t* vals[2] = {(uint32_t*)(ws + ov[0]), (uint32_t*)(ws + ov[1])};
   uint32_t* table = (uint32_t*)(ws + ot);
@@ -316,8 +543,6 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
   const int ntiles = (int)((n_items + RS_TILE - 1) / RS_TILE);
   const uint32_t sentinel = (uint32_t)max_blocks;
 
-  ProfScope ps_("index_build", stream);  // the whole pipeline of small kernels as one record
-  cu_blocks_kernel<<<1, 64, 0, stream>>>(cu_seqlens, batch, block_size, cu_blocks);
   dim3 g_items((unsigned)((n_items + 255) / 256), num_kv_heads);
   make_keys_kernel<<<g_items, 256, 0, stream>>>(topk_idx, topk_stride_h, topk_stride_n, cu_seqlens,
                                                 cu_blocks, batch, n_items, topk, sentinel, keys[0],

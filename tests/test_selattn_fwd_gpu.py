@@ -67,3 +67,32 @@ def test_fwd_matches_oracle(dev, cu, hq, hkv, d, bk, t, dtype):
     print(f"  max|dO|={err_o:.3e} max|dLSE|={err_l:.3e}", flush=True)
     assert err_o <= O_TOL[dtype]
     assert err_l <= LSE_TOL
+
+
+INDEX_CASES = [
+    # cu_seqlens, Hkv, B_K, T
+    ([0, 5000], 2, 64, 16),
+    ([0, 300, 301, 2500, 2500, 4000], 3, 32, 5),      # ragged, an empty and a one-token sequence, odd T
+    ([0, 70000], 1, 16, 8),                          # 4375 blocks: beyond the counting path
+    ([0, 9000], 2, 128, 24),                         # T not a power of two, partial last tile
+]
+
+
+@pytest.mark.parametrize("cu,hkv,bk,t", INDEX_CASES)
+@pytest.mark.parametrize("radix", [False, True])
+def test_index_both_paths(dev, monkeypatch, cu, hkv, bk, t, radix):
+    """The counting path and the radix-sort path of the index build give the same, bit-exact lists."""
+    print(f"case cu={cu} hkv={hkv} bk={bk} t={t} radix={radix}", flush=True)
+    if radix:
+        monkeypatch.setenv("FSA_INDEX_RADIX", "1")
+    else:
+        monkeypatch.delenv("FSA_INDEX_RADIX", raising=False)
+    topk = make_topk_idx(cu, hkv, bk, t, seed=5)
+    # a few out-of-range and padded entries in the middle of rows
+    gen = torch.Generator().manual_seed(6)
+    bad = torch.rand(topk.shape, generator=gen) < 0.02
+    topk = torch.where(bad, torch.full_like(topk, -1), topk)
+    cu_t = torch.tensor(cu, dtype=torch.int32)
+    index = ops.build_index(topk.to(dev), cu_t.to(dev), bk)
+    torch.cuda.synchronize()
+    _check_index(index, topk, cu, bk)
