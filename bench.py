@@ -87,23 +87,49 @@ def cpu_baseline(seq_len: int, d: int, bk: int, topk: int, hkv: int):
     }
 
 
+def _kernel_records(kern, algo):
+    """[{kernel, ms, bound, achieved, peak, unit, frac, algo_tflops, algo_gbs}] sorted by time; `algo` maps a
+    label to (flops, bytes) of one step, or None where no closed form is given (GEMMs of the library etc.)."""
+    out = []
+    for name, ms in sorted(kern.items(), key=lambda kv: -kv[1]):
+        rec = {"kernel": name, "ms": round(ms, 4)}
+        ab = algo.get(name)
+        if ab is not None and ms > 0:
+            fl, by = ab
+            tf, gbs = fl / (ms * 1e-3) / 1e12, by / (ms * 1e-3) / 1e9
+            if tf / MFMA_PEAK_TFLOPS > gbs / HBM_PEAK_GBS:
+                rec.update(bound="mfma", achieved=round(tf, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                           frac=round(tf / MFMA_PEAK_TFLOPS, 4))
+            else:
+                rec.update(bound="hbm", achieved=round(gbs, 2), peak=HBM_PEAK_GBS, unit="GB/s",
+                           frac=round(gbs / HBM_PEAK_GBS, 4))
+            rec.update(algo_tflops=round(tf, 2), algo_gbs=round(gbs, 1))
+        out.append(rec)
+    return out
+
+
 def side_workload(args):
     """Timing of the two parity configurations that are not selected attention alone: the full layer
-    (forward + backward, 4 x 8192 tokens) and one decode step (64 requests).  Same JSON shape, value in ms."""
+    (forward + backward, 4 x 8192 tokens) and one decode step (64 requests).  Same JSON shape, value in ms;
+    every library kernel is listed with its duration and, where its least work has a closed form, with the
+    roofline it sits closer to (algorithmic flops against the MFMA peak, algorithmic bytes against HBM)."""
     import math
     import torch
     from fsa_hip import _lib, ops
     dev = torch.device("cuda:0")
     torch.manual_seed(0)
+    e = 2
+    algo = {}
     if args.workload == "module":
         from fsa.module.fsa import FlashSparseAttention, RopeConfig
-        layer = FlashSparseAttention(hidden_size=4096, num_q_heads=32, num_kv_heads=8, head_dim=128, kernel_size=32,
-                                     kernel_stride=16, block_size=64, topk=16, init_blocks=1, local_blocks=2,
-                                     window_size=512, rope_config=RopeConfig(head_dim=128)).to(dev).to(torch.bfloat16)
-        n = 4 * 8192
-        x = torch.randn(n, 4096, device=dev, dtype=torch.bfloat16, requires_grad=True)
-        w = torch.randn(n, 4096, device=dev, dtype=torch.bfloat16)
-        cu = torch.arange(0, n + 1, 8192, dtype=torch.int32, device=dev)
+        hidden, hq, hkv, d, ks, st, bk, t, win, nseq, slen = 4096, 32, 8, 128, 32, 16, 64, 16, 512, 4, 8192
+        layer = FlashSparseAttention(hidden_size=hidden, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, kernel_size=ks,
+                                     kernel_stride=st, block_size=bk, topk=t, init_blocks=1, local_blocks=2,
+                                     window_size=win, rope_config=RopeConfig(head_dim=d)).to(dev).to(torch.bfloat16)
+        n = nseq * slen
+        x = torch.randn(n, hidden, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        w = torch.randn(n, hidden, device=dev, dtype=torch.bfloat16)
+        cu = torch.arange(0, n + 1, slen, dtype=torch.int32, device=dev)
         name = "FlashSparseAttention layer fwd+bwd, hidden 4096, Hq=32, Hkv=8, D=128, 32/16 compression, B_K=64, " \
                "T=16, window 512, 4 x 8192 tokens"
 
@@ -111,6 +137,50 @@ def side_workload(args):
             layer.zero_grad(set_to_none=True)
             x.grad = None
             (layer(x, cu) * w).sum().backward()
+
+        # least work per kernel label (one step; a label covers every launch of that kernel in the step)
+        g = hq // hkv
+        nc = (slen - ks) // st + 1
+        i = torch.arange(slen)
+        vis_c = int(torch.clamp((i - ks + 1) // st + 1, 0, nc).sum()) * nseq        # (query, compressed key) pairs
+        vis_w = int((torch.clamp(i, max=win) + 1).sum()) * nseq                     # (query, key) pairs of the band
+        with torch.no_grad():
+            _, idx = layer(x, cu, return_topk_idx=True)
+        idx = idx.cpu()
+        ok = idx >= 0
+        pos = torch.arange(slen).repeat(nseq)[None, :, None]
+        lo = idx.long() * bk
+        nkeys = (torch.minimum(pos, lo + bk - 1) - lo + 1).clamp(min=0)
+        pairs = int(ok.sum())                                                        # summed over kv heads
+        p_key = int(torch.where(ok, nkeys, torch.zeros_like(nkeys)).sum())
+        rows = pairs * g
+        qbytes = n * hq * d * e
+        kvbytes = 2 * n * hkv * d * e
+        ckv = 2 * nseq * nc * hkv * d * e
+        algo.update({
+            "selattn_fwd_main": (4.0 * d * p_key * g, rows * (2 * d * e + 4) + kvbytes),
+            "selattn_fwd_reduce": (0.0, rows * (d * e + 4) + n * hq * (d * e + 4)),
+            "selattn_bwd_dqdkdv": (10.0 * d * p_key * g, rows * (3 * d * e + 8) + 2 * kvbytes),
+            "selattn_bwd_dq_reduce": (0.0, rows * d * e + qbytes),
+            "selattn_bwd_delta": (0.0, 2 * qbytes + 4 * n * hq),
+            "cmpattn_bwd_delta": (0.0, 2 * qbytes + 4 * n * hq),
+            "winattn_bwd_delta": (0.0, 2 * qbytes + 4 * n * hq),
+            "cmpattn_fwd": (4.0 * d * vis_c * hq, 2 * qbytes + ckv),
+            "cmpattn_bwd_dq": (6.0 * d * vis_c * hq, 3 * qbytes + ckv),
+            "cmpattn_bwd_dkdv": (8.0 * d * vis_c * hq, 2 * qbytes + 2 * ckv),
+            "winattn_fwd": (4.0 * d * vis_w * hq, 2 * qbytes + kvbytes),
+            "winattn_bwd_dq": (6.0 * d * vis_w * hq, 3 * qbytes + kvbytes),
+            "winattn_bwd_dkdv": (8.0 * d * vis_w * hq, 2 * qbytes + 2 * kvbytes),
+            "cmp_score": (2.0 * d * vis_c * hkv, 4.0 * hkv * n * nc),                # fp32 probabilities written
+            "cmp_topk": (0.0, 4.0 * hkv * n * nc + 4.0 * hkv * n * t),               # ... read back, ids written
+            "rope": (0.0, 2.0 * (2 * qbytes + 2 * n * hkv * d * e + 2 * nseq * nc * hkv * d * e)),  # fwd + bwd, in + out
+            "gate_merge_fwd": (0.0, 4.0 * qbytes),
+            "gate_merge_bwd": (0.0, 7.0 * qbytes),
+            "linear_compress_fwd": (2 * 2.0 * nseq * nc * ks * d * d * hkv, kvbytes + ckv + 2 * hkv * ks * d * d * e),
+            "linear_compress_dx": (2 * 2.0 * nseq * nc * ks * d * d * hkv, kvbytes + ckv + 2 * hkv * ks * d * d * e),
+            "linear_compress_dw": (2 * 2.0 * nseq * nc * ks * d * d * hkv, kvbytes + ckv + 2 * hkv * ks * d * d * 4),
+            "index_build": (0.0, 4.0 * hkv * n * t * 2 + 4.0 * pairs),
+        })
     else:
         hq, hkv, d, bk, t, ks, st, nreq = 32, 8, 128, 64, 16, 32, 16, 64
         gen = torch.Generator().manual_seed(31)
@@ -136,6 +206,13 @@ def side_workload(args):
             idx = ops.decode_topk(raw, lse_c, cu_ck_t, pos, seqlens, hq, ks, st, bk, t, nblk_max,
                                   softmax_scale=1.0 / math.sqrt(d))
             ops.decode_selattn(q, kc, vc, cu_k_t, idx, bk)
+
+        n_vis = sum(min((l - ks) // st + 1, (l - 1 - ks + 1) // st + 1) for l in lens)   # visible compressed keys
+        algo.update({
+            "decode_cmpattn": (4.0 * d * n_vis * hq, 2.0 * n_vis * hkv * d * e),       # K and V rows, once
+            "decode_selattn": (4.0 * d * nreq * t * bk * hq, 2.0 * nreq * t * bk * hkv * d * e),
+            "decode_topk": (0.0, 4.0 * hkv * n_vis),
+        })
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -152,11 +229,15 @@ def side_workload(args):
     kern = {}
     for nm, t_ in recs:
         kern[nm] = kern.get(nm, 0.0) + t_
+    kernels = _kernel_records(kern, algo)
+    lib_ms = sum(kern.values())
     print(json.dumps({"metric": "ms per step", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
                       "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
                       "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
                       "config": {"workload": name},
-                      "library_kernels_ms": {k_: round(v_, 4) for k_, v_ in sorted(kern.items(), key=lambda kv: -kv[1])}}))
+                      "library_kernels_ms_total": round(lib_ms, 4),
+                      "other_ms": round(ms - lib_ms, 4),   # projections on the BLAS library, autograd glue
+                      "kernels": kernels}))
 
 
 def main():
