@@ -49,7 +49,7 @@ constexpr int CMP_BK = 64;      // compressed keys per tile
 constexpr int CMP_ROWS = 128;   // rows per work-group (4 waves x 32)
 
 template <int D> struct CmpLds {
-  static constexpr int KS = D + 8;
+  static constexpr int KS = D + 16;  // 32 B pad: the transposing reads of K^T (dQ kernel) run conflict-free, with 16 B they do not
   static constexpr int VS = D + 16;
   static constexpr int BYTES = (CMP_BK * KS + CMP_BK * VS) * 2;
 };
@@ -68,6 +68,38 @@ __device__ __forceinline__ void stage_kv_tile(const T* kbase, int64_t k_sn, cons
     }
     store16(&Ks[row * KS + col * 8], x);
     if (vbase) store16(&Vs[row * VS + col * 8], y);
+  }
+}
+
+// The same tile in two steps, so that the rows of the next tile travel while the current one is used:
+// kv_tile_load issues the global loads into registers, kv_tile_store parks them in LDS.
+template <typename T, int D> struct KvTileRegs {
+  static constexpr int N = CMP_BK * (D / 8) / 256;  // 16-byte chunks per thread and tensor
+  typename Elem<T>::vec8 k[N], v[N];
+};
+template <typename T, int D>
+__device__ __forceinline__ void kv_tile_load(KvTileRegs<T, D>& r, const T* kbase, int64_t k_sn, const T* vbase,
+                                             int64_t v_sn, int row0, int n_valid, int tid) {
+  typedef typename Elem<T>::vec8 vec8;
+#pragma unroll
+  for (int j = 0; j < KvTileRegs<T, D>::N; ++j) {
+    const int c = tid + 256 * j, row = c / (D / 8), col = c % (D / 8);
+    r.k[j] = zero8<T>();
+    r.v[j] = zero8<T>();
+    if (row < n_valid) {
+      r.k[j] = load16<vec8>(kbase + (int64_t)(row0 + row) * k_sn + col * 8);
+      r.v[j] = load16<vec8>(vbase + (int64_t)(row0 + row) * v_sn + col * 8);
+    }
+  }
+}
+template <typename T, int D>
+__device__ __forceinline__ void kv_tile_store(const KvTileRegs<T, D>& r, T* Ks, T* Vs, int tid) {
+  constexpr int KS = CmpLds<D>::KS, VS = CmpLds<D>::VS;
+#pragma unroll
+  for (int j = 0; j < KvTileRegs<T, D>::N; ++j) {
+    const int c = tid + 256 * j, row = c / (D / 8), col = c % (D / 8);
+    store16(&Ks[row * KS + col * 8], r.k[j]);
+    store16(&Vs[row * VS + col * 8], r.v[j]);
   }
 }
 
@@ -130,9 +162,18 @@ cmpattn_fwd_kernel(CmpParams p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[dt][i] = 0.f;
 
+  constexpr bool PREFETCH = D <= 128;  // the next tile waits in registers where the budget allows
+  KvTileRegs<T, D> nxt;
+  if (PREFETCH && jt0 < n_keys) kv_tile_load<T, D>(nxt, kbase, p.k_sn, vbase, p.v_sn, k0 + jt0, nc - jt0, tid);
   for (int jt = jt0; jt < n_keys; jt += CMP_BK) {
     if (jt != jt0) __syncthreads();
-    stage_kv_tile<T, D>(kbase, p.k_sn, vbase, p.v_sn, k0 + jt, nc - jt, Ks, Vs, tid);
+    if (PREFETCH) {
+      kv_tile_store<T, D>(nxt, Ks, Vs, tid);
+      if (jt + CMP_BK < n_keys)
+        kv_tile_load<T, D>(nxt, kbase, p.k_sn, vbase, p.v_sn, k0 + jt + CMP_BK, nc - jt - CMP_BK, tid);
+    } else {
+      stage_kv_tile<T, D>(kbase, p.k_sn, vbase, p.v_sn, k0 + jt, nc - jt, Ks, Vs, tid);
+    }
     __syncthreads();
     f32x16 acc[NA];
 #pragma unroll
@@ -147,15 +188,24 @@ cmpattn_fwd_kernel(CmpParams p) {
     }
     const int limit = jmax - jt, limit_lo = jmin - jt;
     float mx = m;
+    // tiles that every row of the wave sees completely need no mask
+    const bool full = __all(limit >= CMP_BK - 1 && limit_lo <= 0);
+    if (full) {
 #pragma unroll
-    for (int a = 0; a < NA; ++a)
+      for (int a = 0; a < NA; ++a)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-        const float sv = (key <= limit && key >= limit_lo) ? acc[a][i] : -INFINITY;
-        acc[a][i] = sv;
-        mx = fmaxf(mx, sv);
-      }
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, acc[a][i]);
+    } else {
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+          const float sv = (key <= limit && key >= limit_lo) ? acc[a][i] : -INFINITY;
+          acc[a][i] = sv;
+          mx = fmaxf(mx, sv);
+        }
+    }
     mx = fmaxf(mx, xor32(mx));
     const float mref = (mx == -INFINITY) ? 0.f : mx * p.scale_log2;
     const float alpha = exp2f(m * p.scale_log2 - mref);  // m = -inf -> 0
