@@ -15,6 +15,8 @@
 namespace fsa {
 
 // ------------------------------------------------------------------- rope ----
+// One thread owns 8 + 8 dims (sub, sub + d/2) of one token for all heads: the angles depend on the position and
+// the dim only, so cos / sin are evaluated once per token instead of once per head.
 template <typename T>
 __global__ void __launch_bounds__(256)
 rope_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, T* __restrict__ out, int64_t o_sn,
@@ -23,30 +25,37 @@ rope_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, T* __restrict__
   typedef typename Elem<T>::vec8 vec8;
   const int lpr = d / 16;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t row = idx / lpr;
-  const int sub = (int)(idx - row * lpr);
-  if (row >= n * h) return;
-  const int64_t tok = row / h;
-  const int head = (int)(row - tok * h);
+  const int64_t tok = idx / lpr;
+  const int sub = (int)(idx - tok * lpr);
+  if (tok >= n) return;
   const int s = upper_seg(cu, batch, (int)tok);
   const float pos = (float)(start + ((int)tok - cu[s]) * stride);
-  const T* xr = x + tok * x_sn + (int64_t)head * x_sh + sub * 8;
-  vec8 a = load16<vec8>(xr), b = load16<vec8>(xr + d / 2);
-  vec8 oa, ob;
+  float c[8], sn[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const float ang = pos * inv_freq[sub * 8 + e];
+    float sv, cv;
+    sincosf(ang, &sv, &cv);
     // the tables are rounded to the tensor's dtype before use, as in the reference
-    const float c = (float)(T)(cosf(ang) * attn_scale);
-    float sn = (float)(T)(sinf(ang) * attn_scale);
-    if (conj) sn = -sn;
-    const float x1 = (float)a[e], x2 = (float)b[e];
-    oa[e] = (T)(x1 * c - x2 * sn);
-    ob[e] = (T)(x1 * sn + x2 * c);
+    c[e] = (float)(T)(cv * attn_scale);
+    sn[e] = (float)(T)(sv * attn_scale);
+    if (conj) sn[e] = -sn[e];
   }
-  T* orow = out + tok * o_sn + (int64_t)head * o_sh + sub * 8;
-  store16(orow, oa);
-  store16(orow + d / 2, ob);
+#pragma unroll 4
+  for (int head = 0; head < h; ++head) {
+    const T* xr = x + tok * x_sn + (int64_t)head * x_sh + sub * 8;
+    vec8 a = load16<vec8>(xr), b = load16<vec8>(xr + d / 2);
+    vec8 oa, ob;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float x1 = (float)a[e], x2 = (float)b[e];
+      oa[e] = (T)(x1 * c[e] - x2 * sn[e]);
+      ob[e] = (T)(x1 * sn[e] + x2 * c[e]);
+    }
+    T* orow = out + tok * o_sn + (int64_t)head * o_sh + sub * 8;
+    store16(orow, oa);
+    store16(orow + d / 2, ob);
+  }
 }
 
 // ------------------------------------------------------- linear compress ----
@@ -372,7 +381,7 @@ extern "C" int fsa_rope(const void* x, void* out, int32_t dtype, int64_t x_strid
   FSA_CHECK_ARG(head_dim >= 16 && head_dim % 16 == 0, "fsa_rope: head_dim must be a multiple of 16");
   FSA_CHECK_ARG(batch >= 1 && num_heads >= 1, "fsa_rope: bad sizes");
   if (total_tokens == 0) return 0;
-  const int64_t work = total_tokens * num_heads * (head_dim / 16);
+  const int64_t work = total_tokens * (head_dim / 16);
   const unsigned grid = (unsigned)((work + 255) / 256);
   ProfScope ps_("rope", stream);
   if (dtype == FSA_BF16)
