@@ -255,13 +255,27 @@ decode_merge_kernel(DecParams p, int D) {
     const int col = e / D, d = e - col * D;
     const float* pc = part + col * (2 + D);
     float mt = -INFINITY;
+#pragma unroll 8
     for (int s_ = 0; s_ < ns; ++s_) mt = fmaxf(mt, pc[s_ * slot]);
     float lt = 0.f, o = 0.f;
-    for (int s_ = 0; s_ < ns; ++s_) {
-      const float ms = pc[s_ * slot];
-      const float wgt = ms == -INFINITY ? 0.f : exp2f(ms - mt);
-      lt += wgt * pc[s_ * slot + 1];
-      o += wgt * pc[s_ * slot + 2 + d];
+    // batches of loads issued together; the sums keep the order of the splits
+    constexpr int UB = 8;
+    for (int sb = 0; sb < ns; sb += UB) {
+      float ms[UB], ls[UB], os[UB];
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        const int s_ = min(sb + u, ns - 1);
+        ms[u] = pc[s_ * slot];
+        ls[u] = pc[s_ * slot + 1];
+        os[u] = pc[s_ * slot + 2 + d];
+      }
+#pragma unroll
+      for (int u = 0; u < UB; ++u)
+        if (sb + u < ns) {
+          const float wgt = ms[u] == -INFINITY ? 0.f : exp2f(ms[u] - mt);
+          lt += wgt * ls[u];
+          o += wgt * os[u];
+        }
     }
     const float inv_l = lt > 0.f ? 1.f / lt : 0.f;
     const int hq_i = h * p.g + col;
