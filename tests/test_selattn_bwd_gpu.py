@@ -59,3 +59,59 @@ def test_bwd_matches_oracle(dev, cu, hq, hkv, d, bk, t, dtype, std):
         print(f"  max|d{name}|={err:.3e} (ref max {ref.abs().max().item():.2f})", flush=True)
         excess = ((got - ref).abs() - ULP[dtype] * ref.abs()).max().item()
         assert excess <= TOL[dtype], (name, err, excess)
+
+
+def test_strided_views_and_empty_sequence(dev):
+    """q, k, v (and dO) as head slices of one packed [N, Hq + 2 Hkv, D] buffer, with a zero-length sequence in the
+    batch: the strides reach the kernels as given and the results equal those of contiguous copies bit for bit."""
+    cu, hq, hkv, d, bk, t, dtype = [0, 900, 900, 1500, 2048], 8, 2, 128, 64, 8, torch.bfloat16
+    n = cu[-1]
+    q, k, v, do = make_qkv(n, hq, hkv, d, dtype, seed=17)
+    topk = make_topk_idx(cu, hkv, bk, t, seed=18)
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    packed = torch.cat([q, k, v], dim=1).to(dev)                     # [N, Hq + 2 Hkv, D]
+    qv, kv, vv = packed[:, :hq], packed[:, hq:hq + hkv], packed[:, hq + hkv:]
+    assert not qv.is_contiguous() and not kv.is_contiguous()
+    do_wide = torch.zeros(n, hq + 3, d, dtype=dtype, device=dev)
+    do_wide[:, :hq] = do.to(dev)
+    dov = do_wide[:, :hq]
+    index = ops.build_index(topk.to(dev), cu_t, bk)
+    o1, lse1 = ops.selattn_fwd(qv, kv, vv, index)
+    g1 = ops.selattn_bwd(qv, kv, vv, o1, dov, lse1, index)
+    qc, kc, vc, doc = (x.contiguous() for x in (qv, kv, vv, dov))
+    o2, lse2 = ops.selattn_fwd(qc, kc, vc, index)
+    g2 = ops.selattn_bwd(qc, kc, vc, o2, doc, lse2, index)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2) and torch.equal(lse1, lse2)
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b)
+    o_ref, lse_ref = orc.selected_attention_ref(q.float(), k.float(), v.float(), topk, bk, cu)
+    assert (o1.float().cpu() - o_ref).abs().max().item() <= TOL[dtype]
+    assert (lse1.cpu() - lse_ref).abs().max().item() <= 1e-3
+
+
+def test_query_without_selected_block(dev):
+    """A query whose list holds only padding attends nothing: O = 0, LSE = -inf, dQ = 0 (the reference's kernels give
+    LSE = -inf and an undefined O for such a row, FSA_topk_sparse_attention.py:273); its neighbours are unaffected."""
+    cu, hq, hkv, d, bk, t, dtype = [0, 512], 4, 2, 128, 64, 4, torch.bfloat16
+    n = cu[-1]
+    q, k, v, do = make_qkv(n, hq, hkv, d, dtype, seed=27)
+    topk = make_topk_idx(cu, hkv, bk, t, seed=28)
+    dead = [5, 200, 511]
+    topk[:, dead, :] = -1
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    index = ops.build_index(topk.to(dev), cu_t, bk)
+    qd, kd, vd, dod = (x.to(dev) for x in (q, k, v, do))
+    o, lse = ops.selattn_fwd(qd, kd, vd, index)
+    dq, dk, dv = ops.selattn_bwd(qd, kd, vd, o, dod, lse, index)
+    torch.cuda.synchronize()
+    o, lse, dq = o.float().cpu(), lse.cpu(), dq.float().cpu()
+    assert (o[dead] == 0).all() and torch.isinf(lse[:, dead]).all() and (lse[:, dead] < 0).all()
+    assert (dq[dead] == 0).all()
+    assert torch.isfinite(o).all() and torch.isfinite(dq).all()
+    assert torch.isfinite(dk.float()).all() and torch.isfinite(dv.float()).all()
+    live = torch.ones(n, dtype=torch.bool)
+    live[dead] = False
+    o_ref, lse_ref = orc.selected_attention_ref(q.float(), k.float(), v.float(), topk, bk, cu)
+    assert (o[live] - o_ref[live]).abs().max().item() <= TOL[dtype]
+    assert (lse[:, live] - lse_ref[:, live]).abs().max().item() <= 1e-3
