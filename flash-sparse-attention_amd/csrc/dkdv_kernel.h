@@ -466,7 +466,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
           const int row = lane / CPW + RPI * j;
           const int r = base + rt * 16 + row;
           vec8 x = load16<vec8>(&dQst[row * C::DQS + (lane % CPW) * 8]);
-          if (r < row_hi) store16(dqpart + (prow0 + r) * D + tg * C::DW + (lane % CPW) * 8, x);
+          if (r < row_hi) store16_stream(dqpart + (prow0 + r) * D + tg * C::DW + (lane % CPW) * 8, x);
         }
         __builtin_amdgcn_wave_barrier();
       }

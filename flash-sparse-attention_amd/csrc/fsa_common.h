@@ -54,6 +54,17 @@ template <typename V> __device__ __forceinline__ V load16(const void* p) {
 template <typename V> __device__ __forceinline__ void store16(void* p, V v) {
   *reinterpret_cast<uint4*>(p) = __builtin_bit_cast(uint4, v);
 }
+// The same 16-byte moves for data that is written once and read once by a later kernel (partial rows):
+// marked non-temporal so that they do not displace the K / V blocks and query rows that are reused.
+template <typename V> __device__ __forceinline__ V load16_stream(const void* p) {
+  typedef unsigned int u4_ __attribute__((ext_vector_type(4)));
+  u4_ r = __builtin_nontemporal_load(reinterpret_cast<const u4_*>(p));
+  return __builtin_bit_cast(V, r);
+}
+template <typename V> __device__ __forceinline__ void store16_stream(void* p, V v) {
+  typedef unsigned int u4_ __attribute__((ext_vector_type(4)));
+  __builtin_nontemporal_store(__builtin_bit_cast(u4_, v), reinterpret_cast<u4_*>(p));
+}
 template <typename V> __device__ __forceinline__ V load8(const void* p) {
   uint2 r = *reinterpret_cast<const uint2*>(p);
   return __builtin_bit_cast(V, r);

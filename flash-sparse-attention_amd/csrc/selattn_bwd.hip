@@ -203,7 +203,7 @@ selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __res
     const int pidx = so[t];
     if (pidx < 0) continue;
     const int64_t prow = ((int64_t)kh * cap + pidx) * g + head;
-    vec8 x = load16<vec8>(dq_part + prow * D + sub * 8);
+    vec8 x = load16_stream<vec8>(dq_part + prow * D + sub * 8);
 #pragma unroll
     for (int e = 0; e < 8; ++e) accv[e] += (float)x[e];
   }

@@ -236,7 +236,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
         for (int j = 0; j < 2; ++j) {
           const int row = (lane >> 2) + 16 * j;
           vec8 y = load16<vec8>(&Osl[row * SLS + (lane & 3) * 8]);
-          if (sub + row < row_hi) store16(opart + (prow0 + sub + row) * D + dt * 32 + (lane & 3) * 8, y);
+          if (sub + row < row_hi) store16_stream(opart + (prow0 + sub + row) * D + dt * 32 + (lane & 3) * 8, y);
         }
         __builtin_amdgcn_wave_barrier();
       }
@@ -250,7 +250,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       for (int j = 0; j < 32 / RPI; ++j) {
         const int row = srow + RPI * j;
         vec8 x = load16<vec8>(&Ost[row * OS + schunk * 8]);
-        if (sub + row < row_hi) store16(opart + (prow0 + sub + row) * D + schunk * 8, x);
+        if (sub + row < row_hi) store16_stream(opart + (prow0 + sub + row) * D + schunk * 8, x);
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -319,7 +319,7 @@ selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict_
       if (pidx < 0) continue;
       const int64_t prow = (pbase + pidx) * g + head;
       const float wgt = exp2f(lse_part[prow] - lse_tot);
-      vec8 x = load16<vec8>(o_part + prow * D + sub * 8);
+      vec8 x = load16_stream<vec8>(o_part + prow * D + sub * 8);
 #pragma unroll
       for (int e = 0; e < 8; ++e) accv[e] += wgt * (float)x[e];
     }
