@@ -38,7 +38,7 @@ selattn_bwd_delta_kernel(const T* __restrict__ o, int64_t o_sn, int64_t o_sh,
   if (R >= n_tokens * hq) return;
   const int64_t tok = R / hq;
   const int h = (int)(R - tok * hq);
-  vec8 a = load16<vec8>(o + tok * o_sn + (int64_t)h * o_sh + sub * 8);
+  vec8 a = load16_stream<vec8>(o + tok * o_sn + (int64_t)h * o_sh + sub * 8);
   vec8 b = load16<vec8>(d_o + tok * do_sn + (int64_t)h * do_sh + sub * 8);
   float s = 0.f;
 #pragma unroll
@@ -211,7 +211,7 @@ selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __res
     vec8 out;
 #pragma unroll
     for (int e = 0; e < 8; ++e) out[e] = (T)accv[e];
-    store16(dq + (tok * hq + hq_i) * D + sub * 8, out);
+    store16_stream(dq + (tok * hq + hq_i) * D + sub * 8, out);
     return;
   }
   const int pos = sub * 8;

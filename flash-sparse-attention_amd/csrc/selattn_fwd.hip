@@ -327,7 +327,7 @@ selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict_
   vec8 out;
 #pragma unroll
   for (int e = 0; e < 8; ++e) out[e] = (T)accv[e];
-  store16(o + tok * o_sn + (int64_t)hq_i * o_sh + sub * 8, out);
+  store16_stream(o + tok * o_sn + (int64_t)hq_i * o_sh + sub * 8, out);
   if (sub == 0) lse[(int64_t)hq_i * n_tokens + tok] = lse_tot;
 }
 
