@@ -499,8 +499,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     float* part = p.dkdv_part + ((int64_t)h * p.max_tiles + w) * (2 * BK * D) + key * D + 4 * kg;
 #pragma unroll
     for (int t = 0; t < NDT; ++t) {
-      *reinterpret_cast<f32x4*>(part + 16 * t) = dkacc[t];
-      *reinterpret_cast<f32x4*>(part + BK * D + 16 * t) = dvacc[t];
+      __builtin_nontemporal_store(dkacc[t], reinterpret_cast<f32x4*>(part + 16 * t));
+      __builtin_nontemporal_store(dvacc[t], reinterpret_cast<f32x4*>(part + BK * D + 16 * t));
     }
   }
 }

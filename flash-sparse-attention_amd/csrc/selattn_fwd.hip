@@ -254,7 +254,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       }
     }
     __builtin_amdgcn_wave_barrier();
-    if (valid && hh == 0) p.lse_part[prow] = l > 0.f ? mref + log2f(l) : -INFINITY;
+    if (valid && hh == 0) __builtin_nontemporal_store(l > 0.f ? mref + log2f(l) : -INFINITY, &p.lse_part[prow]);
   };
 
   int sub = row_lo + wv * 32;
