@@ -136,7 +136,7 @@ decode_attn_kernel(DecParams p) {
     for (int j = 0; j < VCH; ++j) {
       const int c = lane + 64 * j, row = c / (D / 8), cc = c % (D / 8);
       vst[j] = zero8<T>();  // rows past n_valid are zero so that 0 * garbage cannot appear
-      if (row < n_valid) vst[j] = load16<vec8>(vbase + (int64_t)(k0 + row0 + row) * p.v_sn + cc * 8);
+      if (row < n_valid) vst[j] = load16_stream<vec8>(vbase + (int64_t)(k0 + row0 + row) * p.v_sn + cc * 8);
     }
     // S^T[key][column] = K Q^T, K fragments straight from global memory
     f32x4 acc[2];
@@ -146,7 +146,7 @@ decode_attn_kernel(DecParams p) {
       const T* krow = kbase + (int64_t)(k0 + row0 + key) * p.k_sn;
       vec8 kf[NS];
 #pragma unroll
-      for (int s_ = 0; s_ < NS; ++s_) kf[s_] = key < n_valid ? load16<vec8>(krow + 32 * s_) : zero8<T>();
+      for (int s_ = 0; s_ < NS; ++s_) kf[s_] = key < n_valid ? load16_stream<vec8>(krow + 32 * s_) : zero8<T>();
 #pragma unroll
       for (int i = 0; i < 4; ++i) acc[a][i] = 0.f;
 #pragma unroll

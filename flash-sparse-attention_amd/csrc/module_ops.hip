@@ -314,7 +314,7 @@ gate_merge_fwd_kernel(const T* __restrict__ a, const T* __restrict__ b, const T*
   const float g0 = (float)gate[n * 3], g1 = (float)gate[n * 3 + 1], g2 = (float)gate[n * 3 + 2];
   const int64_t base = n * row;
   for (int e = lane * 8; e < row; e += 512) {
-    const vec8 x = load16<vec8>(a + base + e), y = load16<vec8>(b + base + e), z = load16<vec8>(c + base + e);
+    const vec8 x = load16_stream<vec8>(a + base + e), y = load16_stream<vec8>(b + base + e), z = load16_stream<vec8>(c + base + e);
     vec8 r;
 #pragma unroll
     for (int i = 0; i < 8; ++i) r[i] = (T)(g0 * (float)x[i] + g1 * (float)y[i] + g2 * (float)z[i]);
@@ -336,8 +336,8 @@ gate_merge_bwd_kernel(const T* __restrict__ d_out, const T* __restrict__ a, cons
   const int64_t base = n * row;
   float s0 = 0.f, s1 = 0.f, s2 = 0.f;
   for (int e = lane * 8; e < row; e += 512) {
-    const vec8 w = load16<vec8>(d_out + base + e);
-    const vec8 x = load16<vec8>(a + base + e), y = load16<vec8>(b + base + e), z = load16<vec8>(c + base + e);
+    const vec8 w = load16_stream<vec8>(d_out + base + e);
+    const vec8 x = load16_stream<vec8>(a + base + e), y = load16_stream<vec8>(b + base + e), z = load16_stream<vec8>(c + base + e);
     vec8 ra, rb, rc;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
