@@ -298,7 +298,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 
     vec4 pk[NRT], dsk[NRT];
     // Q / dO fragments of row tile rt: [Q lo s_ | Q hi s_ | dO lo s_ | dO hi s_], issued one row tile ahead
-    constexpr bool RAW = !KLDS && NS <= 4;
+    constexpr bool RAW = !KLDS && NS <= 4 && C::CPT <= 4;  // where the registers allow it
     constexpr int NF = RAW ? 4 * NS : 1;
     u32x2 fr[2][NF];
     // statistics of the lane's four rows of the tile: [lse 0-1 | lse 2-3 | delta 0-1 | delta 2-3 | limit 0-1 |
