@@ -174,21 +174,26 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 
   // K / V fragments of this wave's 16 keys stay in registers: B[k = d][n = key]
   constexpr bool KLDS = FUSE_DQ && C::K_FROM_LDS;
+  // hand-issued 8-byte fragment reads (and the contraction-index mapping that goes with them) where the
+  // registers allow it
+  constexpr bool SPLIT = !KLDS && NS <= 4 && C::CPT <= 4;
   vec8 kf[KLDS ? 1 : NS], vf[NS];
   {
     // Contraction index of the S / dP products: k-step s_ covers dims [32 s_, 32 s_ + 32); the lane of key
     // group kg holds dims 4 kg .. 4 kg + 3 and 16 + 4 kg .. 16 + 4 kg + 3 of it.  Both halves are 8-byte
     // pieces, so the matching Q / dO fragments come from LDS with 8-byte reads in which the four key groups
     // read 32 contiguous bytes of a row (full LDS rate; a 16-byte read per lane runs at half of it).
-    const T* krow = reinterpret_cast<const T*>(p.k) + (int64_t)ktok * p.k_sn + (int64_t)h * p.k_sh + 4 * kg;
-    const T* vrow = reinterpret_cast<const T*>(p.v) + (int64_t)ktok * p.v_sn + (int64_t)h * p.v_sh + 4 * kg;
+    // (Configurations that keep the compiler-issued 16-byte reads - SPLIT false - use the plain mapping: dims
+    // 8 kg .. 8 kg + 7 of the k-step.)
+    const T* krow = reinterpret_cast<const T*>(p.k) + (int64_t)ktok * p.k_sn + (int64_t)h * p.k_sh + (SPLIT ? 4 : 8) * kg;
+    const T* vrow = reinterpret_cast<const T*>(p.v) + (int64_t)ktok * p.v_sn + (int64_t)h * p.v_sh + (SPLIT ? 4 : 8) * kg;
 #pragma unroll
     for (int s_ = 0; s_ < NS; ++s_) {
       if (!KLDS) kf[s_] = zero8<T>();
       vf[s_] = zero8<T>();
       if (key_ok) {
-        if (!KLDS) kf[s_] = load8x2<T>(krow + 32 * s_);
-        vf[s_] = load8x2<T>(vrow + 32 * s_);
+        if (!KLDS) kf[s_] = SPLIT ? load8x2<T>(krow + 32 * s_) : load16<vec8>(krow + 32 * s_);
+        vf[s_] = SPLIT ? load8x2<T>(vrow + 32 * s_) : load16<vec8>(vrow + 32 * s_);
       }
     }
   }
@@ -280,7 +285,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     }
 
   // lane addresses: A operand rows (natural) and transposing reads
-  const int a_off = l16 * QS + 4 * kg;                            // + rt*16*QS + 32*s (+ 16 for the second half)
+  const int a_off = l16 * QS + (SPLIT ? 4 : 8) * kg;              // + rt*16*QS + 32*s (SPLIT: + 16 for the second half)
   const int tr_off = (4 * kg + (l16 >> 2)) * QS + 4 * (l16 & 3);  // + 32*u*QS + 16*dtile
 
 
@@ -298,7 +303,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 
     vec4 pk[NRT], dsk[NRT];
     // Q / dO fragments of row tile rt: [Q lo s_ | Q hi s_ | dO lo s_ | dO hi s_], issued one row tile ahead
-    constexpr bool RAW = !KLDS && NS <= 4 && C::CPT <= 4;  // where the registers allow it
+    constexpr bool RAW = SPLIT;
     constexpr int NF = RAW ? 4 * NS : 1;
     u32x2 fr[2][NF];
     // statistics of the lane's four rows of the tile: [lse 0-1 | lse 2-3 | delta 0-1 | delta 2-3 | limit 0-1 |
@@ -359,9 +364,9 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       } else {
 #pragma unroll
         for (int s_ = 0; s_ < NS; ++s_) {
-          vec8 qa = load8x2<T>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
-          sacc = Elem<T>::mfma16(qa, KLDS ? load8x2<T>(&Kl[key * C::KS + 32 * s_ + 4 * kg]) : kf[KLDS ? 0 : s_], sacc);
-          vec8 da = load8x2<T>(&Os[rt * 16 * QS + a_off + 32 * s_]);
+          vec8 qa = load16<vec8>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
+          sacc = Elem<T>::mfma16(qa, KLDS ? load16<vec8>(&Kl[key * C::KS + 32 * s_ + 8 * kg]) : kf[KLDS ? 0 : s_], sacc);
+          vec8 da = load16<vec8>(&Os[rt * 16 * QS + a_off + 32 * s_]);
           dpacc = Elem<T>::mfma16(da, vf[s_], dpacc);
           if (C::TIGHT_REGS && (s_ & 1) == 1) asm volatile("" ::: "memory");
         }
