@@ -314,6 +314,28 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     const uint32_t s_addr = lds_addr(lse_s + 4 * kg);
     constexpr int O_BYTES = C::KV_R * QS * 2;  // Os - Qs
     constexpr int STAT_BYTES = C::KV_R * 4;    // del_s - lse_s = lim_s - del_s = llo_s - lim_s
+    // compiler-issued path: k-steps outside, row tiles inside, so that a K fragment that comes from LDS is read
+    // once per pass
+    f32x4 sacc_all[RAW ? 1 : NRT], dpacc_all[RAW ? 1 : NRT];
+    if constexpr (!RAW) {
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt) {
+        sacc_all[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dpacc_all[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int s_ = 0; s_ < NS; ++s_) {
+        const vec8 kfrag = KLDS ? load16<vec8>(&Kl[key * C::KS + 32 * s_ + 8 * kg]) : kf[KLDS ? 0 : s_];
+#pragma unroll
+        for (int rt = 0; rt < NRT; ++rt) {
+          vec8 qa = load16<vec8>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
+          sacc_all[rt] = Elem<T>::mfma16(qa, kfrag, sacc_all[rt]);
+          vec8 da = load16<vec8>(&Os[rt * 16 * QS + a_off + 32 * s_]);
+          dpacc_all[rt] = Elem<T>::mfma16(da, vf[s_], dpacc_all[rt]);
+        }
+        if (C::TIGHT_REGS && (s_ & 1) == 1) asm volatile("" ::: "memory");
+      }
+    }
     auto issue = [&](auto rt_c, u32x2 (&dst)[NF]) {
       constexpr int rt = decltype(rt_c)::value;
       if constexpr (RAW) {
@@ -362,14 +384,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
           dpacc = Elem<T>::mfma16(frag8<T>(cur[2 * NS + s_], cur[3 * NS + s_]), vf[s_], dpacc);
         }
       } else {
-#pragma unroll
-        for (int s_ = 0; s_ < NS; ++s_) {
-          vec8 qa = load16<vec8>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
-          sacc = Elem<T>::mfma16(qa, KLDS ? load16<vec8>(&Kl[key * C::KS + 32 * s_ + 8 * kg]) : kf[KLDS ? 0 : s_], sacc);
-          vec8 da = load16<vec8>(&Os[rt * 16 * QS + a_off + 32 * s_]);
-          dpacc = Elem<T>::mfma16(da, vf[s_], dpacc);
-          if (C::TIGHT_REGS && (s_ & 1) == 1) asm volatile("" ::: "memory");
-        }
+        sacc = sacc_all[rt];
+        dpacc = dpacc_all[rt];
       }
       float lse_r[4], del_r[4];
       int lim_r[4], llo_r[4] = {0, 0, 0, 0};
