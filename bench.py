@@ -28,12 +28,12 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 # (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by the factor that makes the same counter
 # read 1 GiB for the 1 GiB device copy of --calib-copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 PMC_TRAFFIC_BYTES = {
-    ("selattn_bwd_dqdkdv", 4): 14104562688,
-    ("selattn_fwd_main", 4): 8737412096,
-    ("selattn_fwd_main", 2): 4294666240,
-    ("selattn_fwd_main", 1): 2104956928,
-    ("selattn_fwd_reduce", 4): 5298789376,
-    ("selattn_bwd_dq_reduce", 4): 4575891456,
+    ("selattn_bwd_dqdkdv", 4): 13827282937,
+    ("selattn_fwd_main", 4): 8590825932,
+    ("selattn_fwd_main", 2): 4166508921,
+    ("selattn_fwd_main", 1): 2012088454,
+    ("selattn_fwd_reduce", 4): 4989561907,
+    ("selattn_bwd_dq_reduce", 4): 4565568614,
 }
 
 METRIC = "selected-attn fwd+bwd ms & TFLOP/s at 64K, B_K=64, T=16, GQA 1-4; roofline %"
