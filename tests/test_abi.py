@@ -32,7 +32,10 @@ def test_version_and_host_arithmetic():
     assert lib.fsa_version() >= 100
     # tiles upper bound: ceil(N*T*g / rows) + max_blocks
     assert lib.fsa_max_tiles(65536, 16, 1, 1024, 1025) == 65536 * 16 // 1024 + 1025
-    assert lib.fsa_index_workspace_bytes(65536, 16, 4, 1025) >= 4 * 65536 * 16 * 4 * 4
+    # counting path (at most 4095 blocks): one count per (kv head, block or padding bucket, tile of 4096 entries)
+    assert lib.fsa_index_workspace_bytes(65536, 16, 4, 1025) >= 4 * 1026 * (65536 * 16 // 4096) * 4
+    # radix path beyond that: two key and two value buffers of N*T entries per kv head
+    assert lib.fsa_index_workspace_bytes(65536, 16, 4, 4097) >= 4 * 65536 * 16 * 4 * 4
     a = lib.fsa_selattn_fwd_workspace_bytes(65536, 4, 4, 128, 16, 1025)
     b = lib.fsa_selattn_fwd_workspace_bytes(65536, 16, 4, 128, 16, 1025)
     assert b > 3 * a  # partial buffers scale with the GQA group
