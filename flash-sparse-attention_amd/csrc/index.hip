@@ -331,20 +331,25 @@ place_items_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64
   int key[CT_ROUNDS], rank[CT_ROUNDS];
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   int* my_cnt = cnt + w * nbuckets;
+  // all bucket ids first (the loads of every round in flight together), then the ordered ranking
 #pragma unroll
   for (int r = 0; r < CT_ROUNDS; ++r) {
     key[r] = -1;
     rank[r] = 0;
     if (r < rounds) {  // uniform
       const int i = w * per_wave + r * WAVE + lane;
-      const bool ok = r * WAVE + lane < per_wave && i < n_it;
-      int kb = 0;
-      if (ok) {
+      if (r * WAVE + lane < per_wave && i < n_it) {
         const int qi = i / topk, t = i - qi * topk;
-        kb = item_bucket(topk_idx, stride_h, stride_n, cu_seqlens, cu_blocks, batch, h, (int)tok0 + qi, t,
-                         nbuckets - 1);
-        key[r] = kb;
+        key[r] = item_bucket(topk_idx, stride_h, stride_n, cu_seqlens, cu_blocks, batch, h, (int)tok0 + qi, t,
+                             nbuckets - 1);
       }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r) {
+    if (r < rounds) {  // uniform
+      const bool ok = key[r] >= 0;
+      const int kb = ok ? key[r] : 0;
       uint64_t peers = __ballot(ok);
       for (int bit = 0; bit < key_bits; ++bit) {
         const bool one = (kb >> bit) & 1;

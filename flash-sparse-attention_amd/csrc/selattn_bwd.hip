@@ -198,14 +198,20 @@ selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __res
   float accv[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) accv[e] = 0.f;
-#pragma unroll 4
-  for (int t = 0; t < topk; ++t) {
-    const int pidx = so[t];
-    if (pidx < 0) continue;
-    const int64_t prow = ((int64_t)kh * cap + pidx) * g + head;
-    vec8 x = load16_stream<vec8>(dq_part + prow * D + sub * 8);
+  // the LPR lanes of a row split the slots: a slot's position is loaded once by its owner and handed round by
+  // shuffles, so the row loads of a chunk of LPR slots are independent of each other
+  for (int t0 = 0; t0 < topk; t0 += LPR) {
+    const int pidx_mine = t0 + sub < topk ? so[t0 + sub] : -1;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) accv[e] += (float)x[e];
+    for (int j = 0; j < LPR; ++j) {
+      const int pidx = __shfl(pidx_mine, j, LPR);
+      if (pidx >= 0) {
+        const int64_t prow = ((int64_t)kh * cap + pidx) * g + head;
+        vec8 x = load16_stream<vec8>(dq_part + prow * D + sub * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) accv[e] += (float)x[e];
+      }
+    }
   }
   if (natural) {  // partial rows written by the fused kernel are in plain d order
     vec8 out;

@@ -289,9 +289,25 @@ selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict_
   const int32_t* so = slot_of + ((int64_t)kh * n_tokens + tok) * topk;
   const int64_t pbase = (int64_t)kh * cap;
 
-  // pass 1: LSE over the valid slots (lanes of the row split the slots)
+  // The LPR lanes of a row split the slots: lane `sub` owns slots sub, sub + LPR, ...  Position and partial LSE of
+  // a slot are loaded once by their owner and handed to the other lanes by shuffles.
+  constexpr int MAXC = 8;  // chunks of LPR slots kept in registers (topk <= 8 * LPR; more are re-read)
+  const int nchunk = (topk + LPR - 1) / LPR;
+  int pidx_c[MAXC];
+  float lse_c[MAXC];
   float mx = -INFINITY;
-  for (int t = sub; t < topk; t += LPR) {
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    pidx_c[c] = -1;
+    lse_c[c] = -INFINITY;
+    if (c < nchunk) {
+      const int t = c * LPR + sub;
+      if (t < topk) pidx_c[c] = so[t];
+      if (pidx_c[c] >= 0) lse_c[c] = lse_part[(pbase + pidx_c[c]) * g + head];
+      mx = fmaxf(mx, lse_c[c]);
+    }
+  }
+  for (int t = MAXC * LPR + sub; t < topk; t += LPR) {  // beyond the register chunks
     const int pidx = so[t];
     if (pidx >= 0) mx = fmaxf(mx, lse_part[(pbase + pidx) * g + head]);
   }
@@ -299,26 +315,45 @@ selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict_
   for (int o_ = LPR / 2; o_ >= 1; o_ >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o_, LPR));
   float sum = 0.f;
   if (mx > -INFINITY) {
-    for (int t = sub; t < topk; t += LPR) {
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c)
+      if (c < nchunk) sum += fast_exp2(lse_c[c] - mx);  // -inf -> 0
+    for (int t = MAXC * LPR + sub; t < topk; t += LPR) {
       const int pidx = so[t];
-      if (pidx >= 0) sum += exp2f(lse_part[(pbase + pidx) * g + head] - mx);
+      if (pidx >= 0) sum += fast_exp2(lse_part[(pbase + pidx) * g + head] - mx);
     }
   }
 #pragma unroll
   for (int o_ = LPR / 2; o_ >= 1; o_ >>= 1) sum += __shfl_xor(sum, o_, LPR);
   const float lse_tot = sum > 0.f ? mx + log2f(sum) : -INFINITY;
 
-  // pass 2: weighted sum of partial rows
+  // weighted sum of the partial rows
   float accv[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) accv[e] = 0.f;
   if (sum > 0.f) {
-#pragma unroll 4
-    for (int t = 0; t < topk; ++t) {
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+      if (c < nchunk) {  // uniform
+        const float w_mine = fast_exp2(lse_c[c] - lse_tot);  // 0 for padding slots
+#pragma unroll
+        for (int j = 0; j < LPR; ++j) {
+          const int pidx = __shfl(pidx_c[c], j, LPR);
+          const float wgt = __shfl(w_mine, j, LPR);
+          if (pidx >= 0) {
+            const int64_t prow = (pbase + pidx) * g + head;
+            vec8 x = load16_stream<vec8>(o_part + prow * D + sub * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) accv[e] += wgt * (float)x[e];
+          }
+        }
+      }
+    }
+    for (int t = MAXC * LPR; t < topk; ++t) {
       const int pidx = so[t];
       if (pidx < 0) continue;
       const int64_t prow = (pbase + pidx) * g + head;
-      const float wgt = exp2f(lse_part[prow] - lse_tot);
+      const float wgt = fast_exp2(lse_part[prow] - lse_tot);
       vec8 x = load16_stream<vec8>(o_part + prow * D + sub * 8);
 #pragma unroll
       for (int e = 0; e < 8; ++e) accv[e] += wgt * (float)x[e];
