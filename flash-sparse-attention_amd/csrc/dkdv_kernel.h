@@ -94,8 +94,15 @@ template <int MODE, int BK> struct KvBlock {
 };
 
 // ----------------------------------------------------------------- dkdv ----
-constexpr int KV_TILE_ROWS = 4096;   // rows per work-group and head of the group (scaled by g, capped)
-static inline int kv_tile_rows(int g) { return KV_TILE_ROWS * (g < 2 ? g : 2); }
+// Upper bound of the rows one work-group takes from a block (a block with more rows is dealt in equal shares to
+// several work-groups, which then write fp32 dK / dV partials): measured optimum 3072 / 5120 / 8192 rows for GQA
+// groups of 1 / 2 / 4 - smaller tiles balance better, larger ones write fewer partials.
+constexpr int KV_TILE_ROWS_MAX = 8192;
+static inline int kv_tile_rows(int g, int d = 128, int bk = 64) {
+  if (d >= 256 && bk >= 128) return KV_TILE_ROWS_MAX;  // 32-row passes of eight waves: fewer, longer tiles
+  const int r = 1024 + 2048 * g;
+  return r < KV_TILE_ROWS_MAX ? r : KV_TILE_ROWS_MAX;
+}
 
 template <int D, int BK> struct KvCfg {
   static constexpr int NW = BK / 16;        // one wave per 16 keys
@@ -163,8 +170,11 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   const int rows = p.counts[h * p.max_blocks + gb] * p.g;
   const int start = MODE == KV_MODE_SELECTED ? p.starts[h * nbp1 + gb] : 0;
   const int ntile_b = tp[gb + 1] - tp[gb];
-  const int row_lo = (w - tp[gb]) * p.kv_tile_rows;
-  const int row_hi = min(rows, row_lo + p.kv_tile_rows);
+  // the rows of the block are dealt to its work-groups in equal shares (whole passes): a full tile followed by a
+  // short remainder, block after block, would put the long and the short tiles on alternating XCDs
+  const int share = ((rows + ntile_b - 1) / ntile_b + C::KV_R - 1) / C::KV_R * C::KV_R;
+  const int row_lo = (w - tp[gb]) * share;
+  const int row_hi = min(rows, row_lo + share);
 
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int l16 = lane & 15, kg = lane >> 4;

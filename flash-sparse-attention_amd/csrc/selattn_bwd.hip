@@ -245,7 +245,7 @@ static BwdWs bwd_ws_layout(int64_t n, int hq, int hkv, int d, int topk, int bk, 
   const int g = hq / hkv;
   const size_t cap = (size_t)n * topk;
   w.max_tiles_dq = fsa_max_tiles(n, topk, g, DQ_TILE_ROWS, max_blocks);
-  w.max_tiles_kv = fsa_max_tiles(n, topk, g, kv_tile_rows(g), max_blocks);
+  w.max_tiles_kv = fsa_max_tiles(n, topk, g, kv_tile_rows(g, d, bk), max_blocks);
   w.off_delta = 0;
   w.off_dqpart = align_up((size_t)n * hq * 4, 256);
   w.off_tiles_dq = w.off_dqpart + align_up(cap * hkv * g * d * 2, 256);
@@ -401,7 +401,7 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   int32_t* tiles_kv = (int32_t*)(wsp + ws.off_tiles_kv);
   int rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, DQ_TILE_ROWS, tiles_dq, stream_);
   if (rc) return rc;
-  rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, kv_tile_rows(g), tiles_kv, stream_);
+  rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, kv_tile_rows(g, head_dim, block_size), tiles_kv, stream_);
   if (rc) return rc;
 
   const int64_t cap = total_tokens * topk;
@@ -430,7 +430,7 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   p.cu_seqlens_k = nullptr; p.kernel_size = 0; p.kernel_stride = 1;
   SelBwdParams pdq = p, pkv = p;
   pdq.tile_prefix = tiles_dq; pdq.max_tiles = ws.max_tiles_dq; pdq.kv_tile_rows = 0;
-  pkv.tile_prefix = tiles_kv; pkv.max_tiles = ws.max_tiles_kv; pkv.kv_tile_rows = kv_tile_rows(g);
+  pkv.tile_prefix = tiles_kv; pkv.max_tiles = ws.max_tiles_kv; pkv.kv_tile_rows = kv_tile_rows(g, head_dim, block_size);
 
   rc = dtype == FSA_BF16
            ? dispatch_bwd<__bf16>(head_dim, block_size, pdq, pkv, num_kv_heads, ws.max_tiles_dq,

@@ -38,7 +38,16 @@ struct SelFwdParams {
   float* lse_part;
 };
 
-constexpr int SEL_TILE_ROWS = 1024;   // rows per work-group (4 or 8 passes of its waves)
+// Upper bound of the rows one work-group takes from a block (a block with more rows is dealt in equal shares to
+// several work-groups): measured optimum about 3072 / 4096 / 6144-8192 rows for GQA groups of 1 / 2 / 4.
+// Where LDS holds a single work-group per CU (head_dim 256, or 128-key blocks at head_dim 128) 1024 rows balance
+// best.
+static inline int sel_tile_rows(int g, int d, int bk) {
+  const int kv_bytes = (bk * (d + 8) + bk * (d + 16)) * 2, stage_bytes = 32 * (d + 8) * 2;
+  if (kv_bytes + 4 * stage_bytes > 80 * 1024) return 1024;   // SelLds<D, BK>::TWO_WGS is false
+  const int r = 2048 + 1024 * g;
+  return r < 8192 ? r : 8192;
+}
 
 template <int D, int BK> struct SelLds {
   static constexpr int KS = D + 8;   // K row stride in elements (16 B pad: bank spread)
@@ -93,8 +102,11 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   const int tok0 = seq_start + b_local * BK;
   const int rows = p.counts[h * p.max_blocks + gb] * p.g;
   const int start = p.starts[h * nbp1 + gb];
-  const int row_lo = (w - tp[gb]) * SEL_TILE_ROWS;
-  const int row_hi = min(rows, row_lo + SEL_TILE_ROWS);
+  // equal shares of the block's rows (whole passes) for its work-groups
+  const int ntile_b = tp[gb + 1] - tp[gb];
+  const int share = ((rows + ntile_b - 1) / ntile_b + SEL_WG_ROWS - 1) / SEL_WG_ROWS * SEL_WG_ROWS;
+  const int row_lo = (w - tp[gb]) * share;
+  const int row_hi = min(rows, row_lo + share);
 
   const int tid = threadIdx.x;
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
@@ -481,9 +493,9 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
   }
   char* wsp = (char*)workspace;
   int32_t* tile_prefix = (int32_t*)(wsp + ws.off_tiles);
-  int rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, SEL_TILE_ROWS, tile_prefix, stream_);
+  int rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, sel_tile_rows(g, head_dim, block_size), tile_prefix, stream_);
   if (rc) return rc;
-  const int64_t max_tiles = fsa_max_tiles(total_tokens, topk, g, SEL_TILE_ROWS, max_blocks);
+  const int64_t max_tiles = fsa_max_tiles(total_tokens, topk, g, sel_tile_rows(g, head_dim, block_size), max_blocks);
 
   SelFwdParams p;
   p.q = q; p.k = k; p.v = v;
@@ -494,6 +506,7 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
   p.sel_tokens = sel_tokens; p.tile_prefix = tile_prefix;
   p.batch = batch; p.max_blocks = max_blocks; p.cap = total_tokens * topk; p.g = g;
   p.g_shift = group_shift(g);
+
   p.scale_log2 = softmax_scale * LOG2E;
   p.o_part = wsp + ws.off_opart;
   p.lse_part = (float*)(wsp + ws.off_lse);
