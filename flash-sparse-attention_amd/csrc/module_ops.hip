@@ -71,6 +71,21 @@ __device__ __forceinline__ typename Elem<T>::vec8 lds_tr8_rows(const T* p, int s
   return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
+// Forward: a work-group owns 32 compressed tokens of one head; its four waves split the window offsets k
+// (wave w takes k = w, w + 4, ...), each with a private W tile in LDS and no work-group barrier inside the loop,
+// and the four partial Y^T tiles are summed through LDS at the end.  (Few compressed tokens exist - a 16th of
+// the sequence - so the work is spread over the offsets as well to fill the chip.)
+constexpr int LCF_ROWS = 32;  // compressed tokens per work-group
+constexpr int LCF_KC = 32;    // rows of W staged per step and wave
+
+template <int D> struct LcFwdLds {
+  static constexpr int WS = D + 16;                        // W tile row stride (32 B pad for the transposing reads)
+  static constexpr int RS = D + 4;                         // row stride of the fp32 reduction tiles
+  static constexpr int TILE_BYTES = 4 * LCF_KC * WS * 2;
+  static constexpr int RED_BYTES = 4 * LCF_ROWS * RS * 4;
+  static constexpr int BYTES = TILE_BYTES > RED_BYTES ? TILE_BYTES : RED_BYTES;
+};
+
 template <typename T, int D>
 __global__ void __launch_bounds__(256)
 lc_fwd_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __restrict__ w,
@@ -78,15 +93,17 @@ lc_fwd_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __re
               const int32_t* __restrict__ cu_y, int nheads, int ks, int stride) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
-  constexpr int WS = D + 8, NT = D / 32;
-  __shared__ __attribute__((aligned(16))) T Wt[LC_KC * WS];
+  constexpr int WS = LcFwdLds<D>::WS, RS = LcFwdLds<D>::RS, NT = D / 32;
+  constexpr int NLD = LCF_KC * (D / 8) / 64;  // 16-byte chunks of a W tile per lane
+  extern __shared__ __attribute__((aligned(16))) unsigned char lc_smem[];
   const int s = blockIdx.y, h = blockIdx.z;
   const int y0 = cu_y[s], ny = cu_y[s + 1] - y0, x0 = cu_x[s];
-  const int n_lo = blockIdx.x * LC_ROWS;
+  const int n_lo = blockIdx.x * LCF_ROWS;
   if (n_lo >= ny) return;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int col = lane & 31, hh = lane >> 5;
-  const int n = n_lo + wv * 32 + col;
+  T* Wt = reinterpret_cast<T*>(lc_smem) + wv * (LCF_KC * WS);
+  const int n = n_lo + col;
   const bool valid = n < ny;
   const T* xrow0 = x + (int64_t)(x0 + (valid ? n : 0) * stride) * x_sn + (int64_t)h * x_sh + 8 * hh;
   const T* wh = w + (int64_t)h * ks * D * D;
@@ -96,40 +113,61 @@ lc_fwd_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __re
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
-  for (int k = 0; k < ks; ++k)
-    for (int dc = 0; dc < D; dc += LC_KC) {
-      __syncthreads();
-      for (int c = tid; c < LC_KC * (D / 8); c += 256) {
-        const int r = c / (D / 8), cc = c % (D / 8);
-        store16(&Wt[r * WS + cc * 8], load16<vec8>(wh + ((int64_t)k * D + dc + r) * D + cc * 8));
-      }
-      __syncthreads();
+  for (int k = wv; k < ks; k += 4)
+    for (int dc = 0; dc < D; dc += LCF_KC) {
+      vec8 wreg[NLD];
 #pragma unroll
-      for (int kk = 0; kk < LC_KC / 16; ++kk) {
-        vec8 xf = zero8<T>();
-        if (valid) xf = load16<vec8>(xrow0 + (int64_t)k * x_sn + dc + 16 * kk);
+      for (int j = 0; j < NLD; ++j) {
+        const int c = lane + 64 * j, r = c / (D / 8), cc = c % (D / 8);
+        wreg[j] = load16<vec8>(wh + ((int64_t)k * D + dc + r) * D + cc * 8);
+      }
+      vec8 xf[LCF_KC / 16];
+#pragma unroll
+      for (int kk = 0; kk < LCF_KC / 16; ++kk) {
+        xf[kk] = zero8<T>();
+        if (valid) xf[kk] = load16<vec8>(xrow0 + (int64_t)k * x_sn + dc + 16 * kk);
+      }
+      __builtin_amdgcn_wave_barrier();  // the previous tile has been consumed
+#pragma unroll
+      for (int j = 0; j < NLD; ++j) {
+        const int c = lane + 64 * j, r = c / (D / 8), cc = c % (D / 8);
+        store16(&Wt[r * WS + cc * 8], wreg[j]);
+      }
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int kk = 0; kk < LCF_KC / 16; ++kk)
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
           vec8 wf = lds_tr8_rows<T>(&Wt[(16 * kk + 8 * hh + tr_row) * WS + t * 32 + tr_col], WS);
-          acc[t] = Elem<T>::mfma32(wf, xf, acc[t]);
+          acc[t] = Elem<T>::mfma32(wf, xf[kk], acc[t]);
         }
-      }
     }
-  if (!valid) return;
-  T* yrow = y + ((int64_t)(y0 + n) * nheads + h) * D + 4 * hh;
+  // sum of the four waves' tiles: red[wave][row][dout] fp32
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(lc_smem);
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int qd = 0; qd < 4; ++qd) {
-      vec4 v;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        T r = (T)acc[t][4 * qd + e];
-        if (bias) r = (T)((float)r + (float)bias[h * D + t * 32 + 8 * qd + 4 * hh + e]);
-        v[e] = r;
-      }
-      store8(yrow + t * 32 + 8 * qd, v);
+      f32x4 v = {acc[t][4 * qd], acc[t][4 * qd + 1], acc[t][4 * qd + 2], acc[t][4 * qd + 3]};
+      *reinterpret_cast<f32x4*>(&red[(wv * LCF_ROWS + col) * RS + t * 32 + 8 * qd + 4 * hh]) = v;
     }
+  __syncthreads();
+  for (int e = tid; e < LCF_ROWS * (D / 4); e += 256) {
+    const int row = e / (D / 4), d4 = (e % (D / 4)) * 4;
+    if (n_lo + row >= ny) continue;
+    f32x4 sum = *reinterpret_cast<const f32x4*>(&red[row * RS + d4]);
+#pragma unroll
+    for (int ww = 1; ww < 4; ++ww) sum += *reinterpret_cast<const f32x4*>(&red[(ww * LCF_ROWS + row) * RS + d4]);
+    vec4 out;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      T r = (T)sum[i];
+      if (bias) r = (T)((float)r + (float)bias[h * D + d4 + i]);
+      out[i] = r;
+    }
+    store8(y + ((int64_t)(y0 + n_lo + row) * nheads + h) * D + d4, out);
+  }
 }
 
 // bias[h, dout] = sum_{k,d} pe[h,k,d] W[h,k,d,dout]  (fp32 accumulation, rounded once).
@@ -243,7 +281,7 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
              const int32_t* __restrict__ cu_x, const int32_t* __restrict__ cu_y, int batch, int nheads,
              int ks, int stride) {
   typedef typename Elem<T>::vec8 vec8;
-  constexpr int XS = 128 + 8, YS = D + 8, NT = D / 32;
+  constexpr int XS = 128 + 16, YS = D + 16, NT = D / 32;  // 32 B pads: conflict-free transposing reads
   __shared__ __attribute__((aligned(16))) T Xs[LC_KC * XS];
   __shared__ __attribute__((aligned(16))) T Ys[LC_KC * YS];
   const int k = blockIdx.x, h = blockIdx.y, dz = blockIdx.z * 128;
@@ -256,27 +294,44 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
-  for (int n0 = 0; n0 < ny_total; n0 += LC_KC) {
-    __syncthreads();
-    for (int c = tid; c < LC_KC * 16; c += 256) {  // X rows: 128 dims = 16 chunks
-      const int r = c / 16, cc = c % 16;
+  // the rows of the next step travel while the current one is multiplied
+  constexpr int NX = LC_KC * 16 / 256, NY = LC_KC * (D / 8) / 256;
+  vec8 xr[NX], yr[NY];
+  auto load_step = [&](int n0) {
+#pragma unroll
+    for (int j = 0; j < NX; ++j) {  // X rows: 128 dims = 16 chunks
+      const int c = tid + 256 * j, r = c / 16, cc = c % 16;
       const int n = n0 + r;
-      vec8 v = zero8<T>();
+      xr[j] = zero8<T>();
       if (n < ny_total) {
         const int s = upper_seg(cu_y, batch, n);
         const int64_t tok = cu_x[s] + (int64_t)(n - cu_y[s]) * stride + k;
-        v = load16<vec8>(x + tok * x_sn + (int64_t)h * x_sh + dz + cc * 8);
+        xr[j] = load16<vec8>(x + tok * x_sn + (int64_t)h * x_sh + dz + cc * 8);
       }
-      store16(&Xs[r * XS + cc * 8], v);
     }
-    for (int c = tid; c < LC_KC * (D / 8); c += 256) {
-      const int r = c / (D / 8), cc = c % (D / 8);
+#pragma unroll
+    for (int j = 0; j < NY; ++j) {
+      const int c = tid + 256 * j, r = c / (D / 8), cc = c % (D / 8);
       const int n = n0 + r;
-      vec8 v = zero8<T>();
-      if (n < ny_total) v = load16<vec8>(dy + ((int64_t)n * nheads + h) * D + cc * 8);
-      store16(&Ys[r * YS + cc * 8], v);
+      yr[j] = zero8<T>();
+      if (n < ny_total) yr[j] = load16<vec8>(dy + ((int64_t)n * nheads + h) * D + cc * 8);
+    }
+  };
+  load_step(0);
+  for (int n0 = 0; n0 < ny_total; n0 += LC_KC) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NX; ++j) {
+      const int c = tid + 256 * j;
+      store16(&Xs[(c / 16) * XS + (c % 16) * 8], xr[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < NY; ++j) {
+      const int c = tid + 256 * j;
+      store16(&Ys[(c / (D / 8)) * YS + (c % (D / 8)) * 8], yr[j]);
     }
     __syncthreads();
+    if (n0 + LC_KC < ny_total) load_step(n0 + LC_KC);
 #pragma unroll
     for (int kk = 0; kk < LC_KC / 16; ++kk) {
       vec8 xf = lds_tr8_rows<T>(&Xs[(16 * kk + 8 * hh + tr_row) * XS + wv * 32 + tr_col], XS);  // A[m = d][k = n]
@@ -406,12 +461,27 @@ static int lc_fwd_t(const void* x, int64_t x_sn, int64_t x_sh, const void* w, co
     ProfScope ps_("linear_compress_bias", stream);
     lc_bias_kernel<T><<<dim3(h, d / 8), 256, 0, stream>>>((const T*)pe, (const T*)w, (T*)bias, ks * d, d);
   }
-  dim3 grid((unsigned)((max_y + LC_ROWS - 1) / LC_ROWS), batch, h);
-  ProfScope ps_("linear_compress_fwd", stream);
+  dim3 grid((unsigned)((max_y + LCF_ROWS - 1) / LCF_ROWS), batch, h);
   const T* b = pe ? (const T*)bias : nullptr;
-  if (d == 64) lc_fwd_kernel<T, 64><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)w, b, (T*)y, cu_x, cu_y, h, ks, stride);
-  else if (d == 128) lc_fwd_kernel<T, 128><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)w, b, (T*)y, cu_x, cu_y, h, ks, stride);
-  else lc_fwd_kernel<T, 256><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)w, b, (T*)y, cu_x, cu_y, h, ks, stride);
+#define FSA_LC_FWD(DD)                                                                                          \
+  {                                                                                                             \
+    constexpr int lds = LcFwdLds<DD>::BYTES;                                                                    \
+    if (lds > 48 * 1024) {                                                                                      \
+      hipError_t e = hipFuncSetAttribute((const void*)lc_fwd_kernel<T, DD>,                                     \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);                      \
+      if (e != hipSuccess) {                                                                                    \
+        set_error("hipFuncSetAttribute(%d B LDS): %s", lds, hipGetErrorString(e));                              \
+        return (int)e;                                                                                          \
+      }                                                                                                         \
+    }                                                                                                           \
+    ProfScope ps_("linear_compress_fwd", stream);                                                               \
+    lc_fwd_kernel<T, DD><<<grid, 256, lds, stream>>>((const T*)x, x_sn, x_sh, (const T*)w, b, (T*)y, cu_x, cu_y, \
+                                                      h, ks, stride);                                           \
+  }
+  if (d == 64) FSA_LC_FWD(64)
+  else if (d == 128) FSA_LC_FWD(128)
+  else FSA_LC_FWD(256)
+#undef FSA_LC_FWD
   return 0;
 }
 
