@@ -214,21 +214,35 @@ lc_dx_kernel(const T* __restrict__ dy, const T* __restrict__ w, T* __restrict__ 
   for (int i_ = 0; i_ < NT; ++i_)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i_][i] = 0.f;
+  // W[h, k] ([d][dout], 2 D^2 bytes) of the step is staged in LDS: as the A operand every lane reads a different
+  // row of it, which straight from global memory is 64 cache lines per load instruction
+  constexpr int WS = D + 8;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lc_smem[];
+  T* Ws = reinterpret_cast<T*>(lc_smem);
   for (int r = 0; r < nrep; ++r) {
     const int nwin = m - r, k = phase + r * stride;
     const bool ok = valid && nwin >= 0 && nwin < ny;
     const T* dyrow = dy + ((int64_t)(y0 + (ok ? nwin : 0)) * nheads + h) * D + 8 * hh;
-    const T* wk = w + ((int64_t)h * ks + k) * D * D + 8 * hh;
+    const T* wk = w + ((int64_t)h * ks + k) * D * D;
+    vec8 yf[D / 16];
 #pragma unroll
     for (int kk = 0; kk < D / 16; ++kk) {
-      vec8 yf = zero8<T>();
-      if (ok) yf = load16<vec8>(dyrow + 16 * kk);
+      yf[kk] = zero8<T>();
+      if (ok) yf[kk] = load16<vec8>(dyrow + 16 * kk);
+    }
+    if (r) __syncthreads();
+    for (int c = tid; c < D * (D / 8); c += 256) {
+      const int row = c / (D / 8), cc = c % (D / 8);
+      store16(&Ws[row * WS + cc * 8], load16<vec8>(wk + (int64_t)row * D + cc * 8));
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < D / 16; ++kk)
 #pragma unroll
       for (int i_ = 0; i_ < NT; ++i_) {
-        vec8 wf = load16<vec8>(wk + (int64_t)(i_ * 32 + col) * D + 16 * kk);  // A[m = d][k = dout]
-        acc[i_] = Elem<T>::mfma32(wf, yf, acc[i_]);
+        vec8 wf = load16<vec8>(&Ws[(i_ * 32 + col) * WS + 16 * kk + 8 * hh]);  // A[m = d][k = dout]
+        acc[i_] = Elem<T>::mfma32(wf, yf[kk], acc[i_]);
       }
-    }
   }
   if (!valid) return;
   T* xrow = dx + ((int64_t)(x0 + t) * nheads + h) * D + 4 * hh;
@@ -499,12 +513,12 @@ extern "C" int fsa_linear_compress_fwd(const void* x, const void* w, const void*
   FSA_CHECK_ARG(!pe || bias_scratch, "fsa_linear_compress_fwd: bias scratch [H, D] needed with pe");
   if (max_seqlen_y <= 0) return 0;
   hipStream_t stream = (hipStream_t)stream_;
-  if (dtype == FSA_BF16)
-    lc_fwd_t<__bf16>(x, x_stride_n, x_stride_h, w, pe, bias_scratch, y, cu_seqlens_x, cu_seqlens_y, batch,
-                     max_seqlen_y, num_heads, head_dim, kernel_size, kernel_stride, stream);
-  else
-    lc_fwd_t<_Float16>(x, x_stride_n, x_stride_h, w, pe, bias_scratch, y, cu_seqlens_x, cu_seqlens_y, batch,
-                       max_seqlen_y, num_heads, head_dim, kernel_size, kernel_stride, stream);
+  const int rc = dtype == FSA_BF16
+      ? lc_fwd_t<__bf16>(x, x_stride_n, x_stride_h, w, pe, bias_scratch, y, cu_seqlens_x, cu_seqlens_y, batch,
+                         max_seqlen_y, num_heads, head_dim, kernel_size, kernel_stride, stream)
+      : lc_fwd_t<_Float16>(x, x_stride_n, x_stride_h, w, pe, bias_scratch, y, cu_seqlens_x, cu_seqlens_y, batch,
+                           max_seqlen_y, num_heads, head_dim, kernel_size, kernel_stride, stream);
+  if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_linear_compress_fwd");
   return 0;
 }
@@ -518,9 +532,23 @@ static int lc_bwd_t(const void* x, int64_t x_sn, int64_t x_sh, const void* w, co
     const int64_t m_per_phase = (max_x + stride - 1) / stride;
     dim3 grid((unsigned)(stride * ((m_per_phase + LC_ROWS - 1) / LC_ROWS)), batch, h);
     // the grid is sized for the longest sequence; shorter sequences recompute their own tiling inside
-    if (d == 64) lc_dx_kernel<T, 64><<<grid, 256, 0, stream>>>((const T*)dy, (const T*)w, (T*)dx, cu_x, cu_y, h, ks, stride);
-    else if (d == 128) lc_dx_kernel<T, 128><<<grid, 256, 0, stream>>>((const T*)dy, (const T*)w, (T*)dx, cu_x, cu_y, h, ks, stride);
-    else lc_dx_kernel<T, 256><<<grid, 256, 0, stream>>>((const T*)dy, (const T*)w, (T*)dx, cu_x, cu_y, h, ks, stride);
+#define FSA_LC_DX(DD)                                                                                           \
+  {                                                                                                             \
+    constexpr int lds = DD * (DD + 8) * 2;                                                                      \
+    if (lds > 48 * 1024) {                                                                                      \
+      hipError_t e = hipFuncSetAttribute((const void*)lc_dx_kernel<T, DD>,                                      \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds);                      \
+      if (e != hipSuccess) {                                                                                    \
+        set_error("hipFuncSetAttribute(%d B LDS): %s", lds, hipGetErrorString(e));                              \
+        return (int)e;                                                                                          \
+      }                                                                                                         \
+    }                                                                                                           \
+    lc_dx_kernel<T, DD><<<grid, 256, lds, stream>>>((const T*)dy, (const T*)w, (T*)dx, cu_x, cu_y, h, ks, stride); \
+  }
+    if (d == 64) FSA_LC_DX(64)
+    else if (d == 128) FSA_LC_DX(128)
+    else FSA_LC_DX(256)
+#undef FSA_LC_DX
   }
   if (pe) {
     ProfScope ps_("linear_compress_dbias", stream);
@@ -553,12 +581,13 @@ extern "C" int fsa_linear_compress_bwd(const void* x, const void* w, const void*
   FSA_CHECK_ARG(!pe || (dpe && dbias_scratch), "fsa_linear_compress_bwd: dpe and dbias scratch needed with pe");
   FSA_CHECK_ARG(max_seqlen_x >= 1, "fsa_linear_compress_bwd: bad max_seqlen_x");
   hipStream_t stream = (hipStream_t)stream_;
-  if (dtype == FSA_BF16)
-    lc_bwd_t<__bf16>(x, x_stride_n, x_stride_h, w, pe, dy, cu_seqlens_x, cu_seqlens_y, batch, max_seqlen_x, total_y,
-                     num_heads, head_dim, kernel_size, kernel_stride, dx, dw, dpe, dbias_scratch, stream);
-  else
-    lc_bwd_t<_Float16>(x, x_stride_n, x_stride_h, w, pe, dy, cu_seqlens_x, cu_seqlens_y, batch, max_seqlen_x,
-                       total_y, num_heads, head_dim, kernel_size, kernel_stride, dx, dw, dpe, dbias_scratch, stream);
+  const int rc = dtype == FSA_BF16
+      ? lc_bwd_t<__bf16>(x, x_stride_n, x_stride_h, w, pe, dy, cu_seqlens_x, cu_seqlens_y, batch, max_seqlen_x,
+                         total_y, num_heads, head_dim, kernel_size, kernel_stride, dx, dw, dpe, dbias_scratch, stream)
+      : lc_bwd_t<_Float16>(x, x_stride_n, x_stride_h, w, pe, dy, cu_seqlens_x, cu_seqlens_y, batch, max_seqlen_x,
+                           total_y, num_heads, head_dim, kernel_size, kernel_stride, dx, dw, dpe, dbias_scratch,
+                           stream);
+  if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_linear_compress_bwd");
   return 0;
 }
