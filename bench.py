@@ -28,12 +28,14 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 # (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by the factor that makes the same counter
 # read 1 GiB for the 1 GiB device copy of --calib-copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 PMC_TRAFFIC_BYTES = {
-    ("selattn_bwd_dqdkdv", 4): 13827282937,
-    ("selattn_fwd_main", 4): 8590825932,
-    ("selattn_fwd_main", 2): 4166508921,
-    ("selattn_fwd_main", 1): 2012088454,
-    ("selattn_fwd_reduce", 4): 4989561907,
-    ("selattn_bwd_dq_reduce", 4): 4565568614,
+    ("selattn_bwd_dqdkdv", 4): 13537720320,
+    ("selattn_bwd_dqdkdv", 2): 6610281472,
+    ("selattn_bwd_dqdkdv", 1): 3254586368,
+    ("selattn_fwd_main", 4): 8274831360,
+    ("selattn_fwd_main", 2): 4033090560,
+    ("selattn_fwd_main", 1): 1987578880,
+    ("selattn_fwd_reduce", 4): 4978273280,
+    ("selattn_bwd_dq_reduce", 4): 4565579776,
 }
 
 METRIC = "selected-attn fwd+bwd ms & TFLOP/s at 64K, B_K=64, T=16, GQA 1-4; roofline %"
@@ -350,8 +352,8 @@ def main():
             return 0.0, 2 * n * hq * d * e + n * hq * 4
         if name == "index_build":
             return 0.0, 4 * hkv * n * topk * 2 + 4 * (pairs + 2 * nblk * hkv)
-        if name == "selattn_bwd_dkdv_reduce":
-            return 0.0, kv_once
+        # selattn_bwd_dkdv_reduce: no least work of its own - dK / dV written once are counted in the fused
+        # kernel; it only adds up the fp32 partials of blocks that were split over several work-groups
         return 0.0, 0.0
 
     kernels = []
@@ -360,6 +362,9 @@ def main():
         tf, gbs = fl / (ms * 1e-3) / 1e12, by / (ms * 1e-3) / 1e9
         f_mfma, f_hbm = tf / MFMA_PEAK_TFLOPS, gbs / HBM_PEAK_GBS
         rec = {"kernel": name, "gqa": g, "ms": round(ms, 4)}
+        if fl == 0 and by == 0:
+            kernels.append(rec)
+            continue
         if f_mfma > f_hbm:                  # the roofline that binds is the one the kernel sits closer to
             rec.update(bound="mfma", achieved=round(tf, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s", frac=round(f_mfma, 4))
         else:
