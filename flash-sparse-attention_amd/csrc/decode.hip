@@ -8,16 +8,17 @@
 //   decode_topk_kernel: probabilities -> re-binned block scores -> top-k ids.
 //
 // Both attention modes are HBM-bound streams of K/V rows (g rows of queries
-// only).  The keys of a (request, kv head) are split over work-groups of 512
-// keys so that the grid fills the chip whatever the cache lengths are; inside a
-// work-group the four waves take 32-key tiles round-robin: K fragments go
-// straight from global memory into 16x16x32 MFMA operands, the V tile is staged
-// in a wave-private LDS region and read back transposed.  The kernel is kept
-// lean in registers (several waves per SIMD keep enough loads in flight).  The
-// waves' partial (m, l, O) are merged through LDS into one fp32 partial per
-// work-group; a small merge kernel combines the partials of a request in a fixed
-// order.  The query heads occupy the first g of the 16 MFMA columns; column g
-// carries the scoring head.
+// only).  The 32-key tiles of all (request, kv head) pairs form one sequence,
+// and a persistent grid of single-wave work-groups - as many as are resident
+// on the chip at once - cuts it into equal contiguous shares: no work-group is
+// dispatched while the kernel runs, every wave streams for the whole launch
+// and always has the rows of its next tile in flight while it computes the
+// current one.  The rows of a tile arrive row-coalesced (16 B per lane, whole
+// 2*D-byte rows per instruction) and pass through a wave-private LDS tile: K
+// is read back as 16x16x32 MFMA operands, V transposed.  A wave writes one
+// fp32 partial (m, l, O) per pair it touches; a small merge kernel combines
+// the partials of a pair in a fixed order.  The query heads occupy the first
+// g of the 16 MFMA columns; column g carries the scoring head.
 //
 // Semantics: fsa_preview/ops/compressed_attention_decode.py:361-490 (attention),
 // :494-592 (scores), :284-357 (transform), :203-205 (top-k);
@@ -28,8 +29,10 @@ namespace fsa {
 
 constexpr int DEC_MODE_COMPRESSED = 0;
 constexpr int DEC_MODE_SELECTED = 1;
-constexpr int DEC_TK = 32;    // keys per wave tile
-constexpr int DEC_TPS = 16;   // tiles per work-group (512 keys)
+constexpr int DEC_TK = 32;            // keys per wave tile
+constexpr int DEC_MAX_WAVES = 4096;   // upper bound of the persistent grid (the workspace is sized for it)
+// resident waves per SIMD the register budget is set for (head_dim 256 stages twice the rows per tile)
+template <int D> struct DecOcc { static constexpr int WAVES_PER_SIMD = D >= 256 ? 1 : 2; };
 
 struct DecParams {
   const void* q;   // [B, Hq, D]
@@ -47,15 +50,13 @@ struct DecParams {
   int64_t raw_ld;
   int score_head_as_written;  // 0: first head of the group, 1: q-head with the kv head's own index
   int max_keys;             // compressed mode: host upper bound of the visible keys of a request (more are ignored)
-  float* part;              // [B, Hkv, nsplit, g, 2 + D]: base-2 scaled max, sum, unnormalised O
-  int nsplit;
+  float* part;              // [slot][g][4 + D]: base-2 scaled max, sum, 2 unused, unnormalised O
+  int32_t* tile_prefix;     // [B+1]: tiles (over all kv heads) of the requests before b
 };
 
 template <int D> struct DecLds {
   static constexpr int VS = D + 8;
-  static constexpr int WAVE_BYTES = DEC_TK * VS * 2;
-  static constexpr int MERGE_BYTES = 4 * (D * 16 + 32) * 4;
-  static constexpr int BYTES = 4 * WAVE_BYTES > MERGE_BYTES ? 4 * WAVE_BYTES : MERGE_BYTES;
+  static constexpr int BYTES = DEC_TK * VS * 2;  // one wave's tile
 };
 
 // number of 32-key tiles of request b (and, in compressed mode, its visible keys)
@@ -73,192 +74,272 @@ __device__ __forceinline__ int dec_tiles(const DecParams& p, int b, int len, int
   return p.topk * tpb;
 }
 
+// tile_prefix[b] = kv heads x tiles of the requests before b (one wave, scan over the requests)
+template <int MODE>
+__global__ void __launch_bounds__(WAVE)
+decode_plan_kernel(DecParams p) {
+  const int lane = threadIdx.x;
+  int carry = 0;
+  for (int b0 = 0; b0 < p.batch; b0 += WAVE) {
+    const int b = b0 + lane;
+    int nt = 0;
+    if (b < p.batch) {
+      int n_keys, tpb;
+      nt = dec_tiles<MODE>(p, b, p.cu_k[b + 1] - p.cu_k[b], n_keys, tpb) * p.hkv;
+    }
+    int incl = nt;
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+      const int y = __shfl_up(incl, o, WAVE);
+      if (lane >= o) incl += y;
+    }
+    if (b < p.batch) p.tile_prefix[b] = carry + incl - nt;
+    carry += __shfl(incl, WAVE - 1, WAVE);
+  }
+  if (lane == 0) p.tile_prefix[p.batch] = carry;
+}
+
+// Tiles before request b.  Selected mode: every request has topk x tiles-per-block tiles per kv head, so the
+// prefix is a product and the plan kernel is not needed.
+template <int MODE> __device__ __forceinline__ int dec_prefix(const DecParams& p, int b) {
+  if (MODE == DEC_MODE_SELECTED) return b * (p.topk * ((p.block_size + DEC_TK - 1) / DEC_TK) * p.hkv);
+  return p.tile_prefix[b];
+}
+// request that holds tile x of the sequence (x < total)
+template <int MODE> __device__ __forceinline__ int dec_request_of(const DecParams& p, int x) {
+  if (MODE == DEC_MODE_SELECTED) return x / (p.topk * ((p.block_size + DEC_TK - 1) / DEC_TK) * p.hkv);
+  return upper_seg(p.tile_prefix, p.batch, x);
+}
+
+// share of the tile sequence per wave for a grid of n_waves
+__device__ __forceinline__ int dec_share(int total, int n_waves) { return max(1, (total + n_waves - 1) / n_waves); }
+
 template <typename T, int D, int MODE>
-__global__ void __launch_bounds__(256, 2)
+__global__ void __launch_bounds__(WAVE, DecOcc<D>::WAVES_PER_SIMD)
 decode_attn_kernel(DecParams p) {
   typedef typename Elem<T>::vec8 vec8;
   constexpr int VS = DecLds<D>::VS;
-  constexpr int NS = D / 32, NDT = D / 16, VCH = DEC_TK * (D / 8) / 64;
+  constexpr int NS = D / 32, NDT = D / 16, VCH = DEC_TK * (D / 8) / 64, PS = D + 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // kv heads vary fastest over the grid: work-groups that run together read neighbouring 2*D-byte pieces of the
-  // same cache rows
-  const int h = blockIdx.x, split = blockIdx.y, b = blockIdx.z;
-  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-  const int l16 = lane & 15, kg = lane >> 4;
-  T* Vs = reinterpret_cast<T*>(smem) + wv * (DEC_TK * VS);
+  T* Vs = reinterpret_cast<T*>(smem);
+  const int lane = threadIdx.x, l16 = lane & 15, kg = lane >> 4;
+  const int w = blockIdx.x;
+  const int total = dec_prefix<MODE>(p, p.batch);
+  const int per = dec_share(total, gridDim.x);
+  const int x_lo = w * per, x_hi = min(total, x_lo + per);
+  if (x_lo >= x_hi) return;
 
-  const int k0 = p.cu_k[b], len = p.cu_k[b + 1] - k0;
-  int n_keys, tpb;
-  const int n_tiles = dec_tiles<MODE>(p, b, len, n_keys, tpb);
-  const int t_lo = split * DEC_TPS;
-  if (t_lo >= n_tiles) return;  // the merge kernel derives the number of live splits the same way
-  const int t_hi = min(n_tiles, t_lo + DEC_TPS);
-  const int32_t* sel = MODE == DEC_MODE_SELECTED ? p.topk_idx + ((int64_t)h * p.batch + b) * p.topk : nullptr;
-
+  // position in the tile sequence: request (with its sizes), kv head, tile of the pair
+  struct Req { int b, k0, len, n_keys, tpb, nt; };
+  auto load_req = [&](Req& r, int b) {
+    r.b = b;
+    r.k0 = p.cu_k[b];
+    r.len = p.cu_k[b + 1] - r.k0;
+    r.nt = dec_tiles<MODE>(p, b, r.len, r.n_keys, r.tpb);
+  };
+  // first cache row and number of valid keys (0: nothing to do) of a tile
+  auto tile_desc = [&](const Req& r, int h, int tt, int& row0, int& n_valid) {
+    if (MODE == DEC_MODE_COMPRESSED) {
+      row0 = tt * DEC_TK;
+      n_valid = min(DEC_TK, r.n_keys - row0);
+    } else {
+      const int32_t* sel = p.topk_idx + ((int64_t)h * p.batch + r.b) * p.topk;
+      const int t = tt / r.tpb, sub = tt - t * r.tpb;
+      const int blk = sel[t];
+      bool dup = false;
+      for (int u = 0; u < t; ++u) dup |= sel[u] == blk;
+      row0 = blk * p.block_size + sub * DEC_TK;
+      n_valid = (blk < 0 || dup) ? 0 : min(min(DEC_TK, p.block_size - sub * DEC_TK), r.len - row0);
+    }
+    n_valid = max(n_valid, 0);
+    row0 = n_valid > 0 ? row0 : 0;
+  };
+  // rows of a tile, coalesced (16 B per lane, D/8 lanes per row); rows past n_valid are zero so that
+  // 0 * garbage cannot appear
+  // (the offsets inside a tile fit 32 bits: uniform base pointer + one offset register per lane)
+  auto load_tile = [&](vec8 (&dst)[VCH], const T* base, int64_t sn, int n_valid) {
+    constexpr int RPI = 64 / (D / 8);  // rows per load instruction
+    const uint32_t off0 = (uint32_t)(lane / (D / 8)) * (uint32_t)sn + (uint32_t)(lane % (D / 8)) * 8u;
+    const uint32_t step = (uint32_t)RPI * (uint32_t)sn;
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int row = lane / (D / 8) + RPI * j;
+      dst[j] = zero8<T>();
+      if (row < n_valid) dst[j] = load16_stream<vec8>(base + (off0 + step * (uint32_t)j));
+    }
+  };
+  auto park_tile = [&](const vec8 (&src)[VCH]) {
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int c = lane + 64 * j, row = c / (D / 8), cc = c % (D / 8);
+      store16(&Vs[row * VS + cc * 8], src[j]);
+    }
+  };
   // B operand [k = d][n = column]: columns 0..g-1 = heads of the group, column g = scoring head (compressed mode)
   vec8 qreg[NS];
-  {
+  auto load_q = [&](int b, int h) {
     int hq_i = -1;
     if (l16 < p.g) hq_i = h * p.g + l16;
     else if (MODE == DEC_MODE_COMPRESSED && l16 == p.g) hq_i = p.score_head_as_written ? h : h * p.g;
     const T* qrow = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)max(hq_i, 0) * p.q_sh + 8 * kg;
 #pragma unroll
     for (int s_ = 0; s_ < NS; ++s_) qreg[s_] = hq_i >= 0 ? load16<vec8>(qrow + 32 * s_) : zero8<T>();
-  }
-  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh + 8 * kg;
-  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
+  };
+  const T* kall = reinterpret_cast<const T*>(p.k);
+  const T* vall = reinterpret_cast<const T*>(p.v);
   const T* vtr = Vs + (4 * kg + (l16 >> 2)) * VS + 4 * (l16 & 3);
 
   float m = -INFINITY, l = 0.f;  // of column l16, replicated over the four key groups
   f32x4 oacc[NDT];               // O^T[d = 16 t + 4 kg + i][column l16]
 #pragma unroll
-  for (int t = 0; t < NDT; ++t)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) oacc[t][i] = 0.f;
+  for (int t = 0; t < NDT; ++t) oacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int tt = t_lo + wv; tt < t_hi; tt += 4) {
-    int row0, n_valid;
-    if (MODE == DEC_MODE_COMPRESSED) {
-      row0 = tt * DEC_TK;
-      n_valid = min(DEC_TK, n_keys - row0);
-    } else {
-      const int t = tt / tpb, sub = tt - t * tpb;
-      const int blk = sel[t];
-      bool dup = false;
-      for (int u = 0; u < t; ++u) dup |= sel[u] == blk;
-      row0 = blk * p.block_size + sub * DEC_TK;
-      n_valid = (blk < 0 || dup) ? 0 : min(min(DEC_TK, p.block_size - sub * DEC_TK), len - row0);
+  Req rq, rqn;
+  load_req(rq, dec_request_of<MODE>(p, x_lo));
+  int h, tt;
+  {
+    const int rem = x_lo - dec_prefix<MODE>(p, rq.b);
+    h = rem / rq.nt;
+    tt = rem - h * rq.nt;
+  }
+  rqn = rq;
+  int hn = h, ttn = tt;
+  int row0, n_valid;
+  tile_desc(rq, h, tt, row0, n_valid);
+  vec8 kst[VCH], vst[VCH];
+  load_tile(kst, kall + (int64_t)(rq.k0 + row0) * p.k_sn + (int64_t)h * p.k_sh, p.k_sn, n_valid);
+  load_tile(vst, vall + (int64_t)(rq.k0 + row0) * p.v_sn + (int64_t)h * p.v_sh, p.v_sn, n_valid);
+  load_q(rq.b, h);
+
+  for (int x = x_lo; x < x_hi; ++x) {
+    const bool has_next = x + 1 < x_hi;
+    int row0n = 0, n_validn = 0;
+    if (has_next) {  // x + 1 < total: a further tile exists
+      if (++ttn == rqn.nt) {
+        ttn = 0;
+        if (++hn == p.hkv) {
+          hn = 0;
+          do load_req(rqn, rqn.b + 1); while (rqn.nt == 0);
+        }
+      }
+      tile_desc(rqn, hn, ttn, row0n, n_validn);
     }
-    if (n_valid <= 0) continue;  // uniform per wave
-    // V rows (coalesced, 16 B per lane) are requested first so that they travel while S is computed
-    vec8 vst[VCH];
-#pragma unroll
-    for (int j = 0; j < VCH; ++j) {
-      const int c = lane + 64 * j, row = c / (D / 8), cc = c % (D / 8);
-      vst[j] = zero8<T>();  // rows past n_valid are zero so that 0 * garbage cannot appear
-      if (row < n_valid) vst[j] = load16_stream<vec8>(vbase + (int64_t)(k0 + row0 + row) * p.v_sn + cc * 8);
-    }
-    // S^T[key][column] = K Q^T, K fragments straight from global memory
-    f32x4 acc[2];
-#pragma unroll
-    for (int a = 0; a < 2; ++a) {
-      const int key = a * 16 + l16;
-      const T* krow = kbase + (int64_t)(k0 + row0 + key) * p.k_sn;
-      vec8 kf[NS];
-#pragma unroll
-      for (int s_ = 0; s_ < NS; ++s_) kf[s_] = key < n_valid ? load16_stream<vec8>(krow + 32 * s_) : zero8<T>();
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[a][i] = 0.f;
-#pragma unroll
-      for (int s_ = 0; s_ < NS; ++s_) acc[a] = Elem<T>::mfma16(kf[s_], qreg[s_], acc[a]);
-    }
-    if (MODE == DEC_MODE_COMPRESSED && p.raw_score && l16 == p.g) {
-      float* rs = p.raw_score + ((int64_t)h * p.batch + b) * p.raw_ld + row0;
+    const bool live = n_valid > 0;  // uniform
+    // the K rows go through the LDS tile first, V uses it afterwards; the rows of the next tile are requested as
+    // soon as the staging registers are free, so that they travel while this tile is computed
+    if (live) park_tile(kst);
+    load_tile(kst, kall + (int64_t)(rqn.k0 + row0n) * p.k_sn + (int64_t)hn * p.k_sh, p.k_sn, n_validn);
+    float alpha = 1.f;
+    vec8 pk = zero8<T>();  // contraction index 8 kg + j  <->  key 4 kg + j (j < 4), 16 + 4 kg + j - 4 (j >= 4)
+    if (live) {
+      __builtin_amdgcn_wave_barrier();
+      // S^T[key][column] = K Q^T
+      f32x4 acc[2];
 #pragma unroll
       for (int a = 0; a < 2; ++a) {
-        const int key0 = a * 16 + 4 * kg;
-        if (row0 + key0 < p.raw_ld) *reinterpret_cast<f32x4*>(rs + key0) = acc[a];
+        acc[a] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s_ = 0; s_ < NS; ++s_) {
+          vec8 kf = load16<vec8>(&Vs[(a * 16 + l16) * VS + 32 * s_ + 8 * kg]);
+          acc[a] = Elem<T>::mfma16(kf, qreg[s_], acc[a]);
+        }
       }
-    }
-    float mx = m;
+      __builtin_amdgcn_wave_barrier();
+      if (MODE == DEC_MODE_COMPRESSED && p.raw_score && l16 == p.g) {
+        float* rs = p.raw_score + ((int64_t)h * p.batch + rq.b) * p.raw_ld + row0;
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = a * 16 + 4 * kg + i;
-        const float sv = key < n_valid ? acc[a][i] : -INFINITY;
-        acc[a][i] = sv;
-        mx = fmaxf(mx, sv);
+        for (int a = 0; a < 2; ++a) {
+          const int key0 = a * 16 + 4 * kg;
+          if (row0 + key0 < p.raw_ld) *reinterpret_cast<f32x4*>(rs + key0) = acc[a];
+        }
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float mref = mx * p.scale_log2;  // n_valid > 0, so mx is finite
-    const float alpha = exp2f(m * p.scale_log2 - mref);
-    float lsum = 0.f;
-    vec8 pk;  // contraction index 8 kg + j  <->  key 4 kg + j (j < 4), 16 + 4 kg + j - 4 (j >= 4)
+      float mx = m;
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < 2; ++a)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float pv = fast_exp2(acc[a][i] * p.scale_log2 - mref);
-        lsum += pv;
-        pk[a * 4 + i] = (T)pv;
+        for (int i = 0; i < 4; ++i) {
+          const int key = a * 16 + 4 * kg + i;
+          const float sv = key < n_valid ? acc[a][i] : -INFINITY;
+          acc[a][i] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float mref = mx * p.scale_log2;  // n_valid > 0, so mx is finite
+      alpha = exp2f(m * p.scale_log2 - mref);
+      float lsum = 0.f;
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float pv = fast_exp2(acc[a][i] * p.scale_log2 - mref);
+          lsum += pv;
+          pk[a * 4 + i] = (T)pv;
+        }
+      lsum += __shfl_xor(lsum, 16, 64);
+      lsum += __shfl_xor(lsum, 32, 64);
+      l = l * alpha + lsum;
+      m = mx;
+      park_tile(vst);
+    }
+    load_tile(vst, vall + (int64_t)(rqn.k0 + row0n) * p.v_sn + (int64_t)hn * p.v_sh, p.v_sn, n_validn);
+    if (live) {
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int t = 0; t < NDT; ++t) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) oacc[t][i] *= alpha;
+        vec8 vf = lds_read_tr8<T>(vtr + 16 * t, 16 * VS);  // V^T[d = 16 t + l16][keys in the order of pk]
+        oacc[t] = Elem<T>::mfma16(vf, pk, oacc[t]);
       }
-    lsum += __shfl_xor(lsum, 16, 64);
-    lsum += __shfl_xor(lsum, 32, 64);
-    l = l * alpha + lsum;
-    m = mx;
-#pragma unroll
-    for (int j = 0; j < VCH; ++j) {
-      const int c = lane + 64 * j, row = c / (D / 8), cc = c % (D / 8);
-      store16(&Vs[row * VS + cc * 8], vst[j]);
+      __builtin_amdgcn_wave_barrier();
     }
-    __builtin_amdgcn_wave_barrier();
+    if (!has_next || hn != h || rqn.b != rq.b) {
+      // last tile of the pair in this wave's share: the partial of (wave, pair) goes to slot wave + pair, which
+      // no other (wave, pair) can name because the shares are contiguous
+      float* out = p.part + (int64_t)(w + rq.b * p.hkv + h) * (p.g * PS);
+      if (l16 < p.g) {
+        float* oc = out + l16 * PS;
+        if (kg == 0) *reinterpret_cast<f32x4*>(oc) = f32x4{m * p.scale_log2, l, 0.f, 0.f};
 #pragma unroll
-    for (int t = 0; t < NDT; ++t) {
+        for (int t = 0; t < NDT; ++t) *reinterpret_cast<f32x4*>(oc + 4 + 16 * t + 4 * kg) = oacc[t];
+      }
+      m = -INFINITY;
+      l = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) oacc[t][i] *= alpha;
-      vec8 vf = lds_read_tr8<T>(vtr + 16 * t, 16 * VS);  // V^T[d = 16 t + l16][keys in the order of pk]
-      oacc[t] = Elem<T>::mfma16(vf, pk, oacc[t]);
+      for (int t = 0; t < NDT; ++t) oacc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (has_next) load_q(rqn.b, hn);
     }
-    __builtin_amdgcn_wave_barrier();
-  }
-
-  // merge the four waves through LDS, then one fp32 partial per work-group
-  __syncthreads();
-  float* mg = reinterpret_cast<float*>(smem);
-  constexpr int PER = D * 16 + 32;
-  float* mine = mg + wv * PER;
-  if (kg == 0) {
-    mine[l16] = m * p.scale_log2;
-    mine[16 + l16] = l;
-  }
-#pragma unroll
-  for (int t = 0; t < NDT; ++t)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) mine[32 + (16 * t + 4 * kg + i) * 16 + l16] = oacc[t][i];
-  __syncthreads();
-  float* out = p.part + (((int64_t)b * p.hkv + h) * p.nsplit + split) * (p.g * (2 + D));
-  for (int e = tid; e < p.g * D; e += 256) {
-    const int col = e / D, d = e - col * D;
-    float mt = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) mt = fmaxf(mt, mg[w * PER + col]);
-    float lt = 0.f, o = 0.f;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const float mw = mg[w * PER + col];
-      const float wgt = mw == -INFINITY ? 0.f : exp2f(mw - mt);
-      lt += wgt * mg[w * PER + 16 + col];
-      o += wgt * mg[w * PER + 32 + d * 16 + col];
-    }
-    out[col * (2 + D) + 2 + d] = o;
-    if (d == 0) {
-      out[col * (2 + D)] = mt;
-      out[col * (2 + D) + 1] = lt;
-    }
+    rq = rqn;
+    h = hn;
+    tt = ttn;
+    row0 = row0n;
+    n_valid = n_validn;
   }
 }
 
-// partials of a request -> o, lse (fixed order over the splits)
+// partials of a pair -> o, lse (fixed order over the waves that shared its tiles)
 template <typename T, int MODE>
 __global__ void __launch_bounds__(256)
-decode_merge_kernel(DecParams p, int D) {
+decode_merge_kernel(DecParams p, int D, int n_waves) {
   const int b = blockIdx.x, h = blockIdx.y;
   const int len = p.cu_k[b + 1] - p.cu_k[b];
   int n_keys, tpb;
-  const int n_tiles = dec_tiles<MODE>(p, b, len, n_keys, tpb);
-  const int ns = (n_tiles + DEC_TPS - 1) / DEC_TPS;
-  const int slot = p.g * (2 + D);
-  const float* part = p.part + ((int64_t)b * p.hkv + h) * p.nsplit * slot;
+  const int nt = dec_tiles<MODE>(p, b, len, n_keys, tpb);
+  const int per = dec_share(dec_prefix<MODE>(p, p.batch), n_waves);
+  const int x0 = dec_prefix<MODE>(p, b) + h * nt;
+  const int w0 = x0 / per;
+  const int ns = nt > 0 ? (x0 + nt - 1) / per - w0 + 1 : 0;
+  const int PS = D + 4, slot = p.g * PS;
+  const float* part = p.part + (int64_t)(w0 + b * p.hkv + h) * slot;
   for (int e = threadIdx.x; e < p.g * D; e += 256) {
     const int col = e / D, d = e - col * D;
-    const float* pc = part + col * (2 + D);
+    const float* pc = part + col * PS;
     float mt = -INFINITY;
 #pragma unroll 8
     for (int s_ = 0; s_ < ns; ++s_) mt = fmaxf(mt, pc[s_ * slot]);
     float lt = 0.f, o = 0.f;
-    // batches of loads issued together; the sums keep the order of the splits
+    // batches of loads issued together; the sums keep the order of the waves
     constexpr int UB = 8;
     for (int sb = 0; sb < ns; sb += UB) {
       float ms[UB], ls[UB], os[UB];
@@ -267,7 +348,7 @@ decode_merge_kernel(DecParams p, int D) {
         const int s_ = min(sb + u, ns - 1);
         ms[u] = pc[s_ * slot];
         ls[u] = pc[s_ * slot + 1];
-        os[u] = pc[s_ * slot + 2 + d];
+        os[u] = pc[s_ * slot + 4 + d];
       }
 #pragma unroll
       for (int u = 0; u < UB; ++u)
@@ -384,20 +465,40 @@ decode_topk_kernel(DecTopkParams p) {
   }
 }
 
+// number of single-wave work-groups that are resident at once on the current device
+template <typename T, int D, int MODE>
+static int dec_grid_waves(int* n_waves) {
+  static int cached[16] = {0};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess && dev >= 0 && dev < 16 && cached[dev] > 0) {
+    *n_waves = cached[dev];
+    return 0;
+  }
+  int cus = 0, per_cu = 0;
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess)
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_attn_kernel<T, D, MODE>, WAVE, DecLds<D>::BYTES);
+  if (e != hipSuccess || cus < 1 || per_cu < 1) {
+    set_error("decode: occupancy query failed (%s, %d CUs, %d work-groups per CU)", hipGetErrorString(e), cus, per_cu);
+    return e != hipSuccess ? (int)e : FSA_ERR_UNSUPPORTED;
+  }
+  int n = cus * per_cu;
+  if (n > DEC_MAX_WAVES) n = DEC_MAX_WAVES;
+  if (dev >= 0 && dev < 16) cached[dev] = n;
+  *n_waves = n;
+  return 0;
+}
+
 template <typename T, int D, int MODE>
 static int dec_launch(const DecParams& p, hipStream_t stream) {
-  constexpr int lds = DecLds<D>::BYTES;
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)decode_attn_kernel<T, D, MODE>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(%d B LDS): %s", lds, hipGetErrorString(e));
-      return (int)e;
-    }
-  }
+  int n_waves = 0;
+  int rc = dec_grid_waves<T, D, MODE>(&n_waves);
+  if (rc) return rc;
   ProfScope ps_(MODE == DEC_MODE_COMPRESSED ? "decode_cmpattn" : "decode_selattn", stream);
-  if (p.nsplit > 0) decode_attn_kernel<T, D, MODE><<<dim3(p.hkv, p.nsplit, p.batch), 256, lds, stream>>>(p);
-  decode_merge_kernel<T, MODE><<<dim3(p.batch, p.hkv), 256, 0, stream>>>(p, D);
+  if (MODE == DEC_MODE_COMPRESSED) decode_plan_kernel<MODE><<<1, WAVE, 0, stream>>>(p);
+  decode_attn_kernel<T, D, MODE><<<n_waves, WAVE, DecLds<D>::BYTES, stream>>>(p);
+  decode_merge_kernel<T, MODE><<<dim3(p.batch, p.hkv), 256, 0, stream>>>(p, D, n_waves);
   return 0;
 }
 
@@ -416,12 +517,10 @@ static int dec_dispatch(int dtype, int head_dim, const DecParams& p, hipStream_t
   return FSA_ERR_UNSUPPORTED;
 }
 
-static int dec_splits(int64_t max_keys) {
-  const int64_t tiles = (max_keys + DEC_TK - 1) / DEC_TK;
-  return (int)((tiles + DEC_TPS - 1) / DEC_TPS);
-}
-static size_t dec_ws_bytes(int batch, int hq, int hkv, int d, int64_t max_keys) {
-  return (size_t)batch * hkv * (size_t)(dec_splits(max_keys) > 0 ? dec_splits(max_keys) : 1) * (hq / hkv) * (2 + d) * 4;
+// workspace: tile prefix of the requests, then one partial slot per (wave, pair) that can occur
+static size_t dec_ws_prefix_bytes(int batch) { return align_up((size_t)(batch + 1) * 4, 256); }
+static size_t dec_ws_bytes(int batch, int hq, int hkv, int d) {
+  return dec_ws_prefix_bytes(batch) + ((size_t)DEC_MAX_WAVES + (size_t)batch * hkv) * (hq / hkv) * (4 + d) * 4;
 }
 
 }  // namespace fsa
@@ -431,7 +530,7 @@ using namespace fsa;
 extern "C" size_t fsa_decode_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
                                              int32_t head_dim, int64_t max_keys) {
   if (batch < 1 || num_kv_heads < 1 || num_q_heads % num_kv_heads || max_keys < 0) return 0;
-  return dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_keys);
+  return dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim);
 }
 
 extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv, int32_t dtype,
@@ -450,7 +549,7 @@ extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv,
   const int g = num_q_heads / num_kv_heads;
   FSA_CHECK_ARG(g <= 15, "fsa_decode_cmpattn: at most 15 query heads per kv head");
   FSA_CHECK_ARG(max_keys >= 0 && max_keys < (1ll << 30), "fsa_decode_cmpattn: bad max_keys");
-  FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_keys),
+  FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim),
                 "fsa_decode_cmpattn: workspace too small (see fsa_decode_workspace_bytes)");
   FSA_CHECK_ARG(batch >= 1 && kernel_size >= 1 && kernel_stride >= 1, "fsa_decode_cmpattn: bad sizes");
   FSA_CHECK_ARG(!raw_score || (raw_ld >= 4 && raw_ld % 4 == 0), "fsa_decode_cmpattn: raw_ld must be a multiple of 4");
@@ -462,7 +561,8 @@ extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv,
   p.kernel_size = kernel_size; p.kernel_stride = kernel_stride; p.scale_log2 = softmax_scale * LOG2E;
   p.o = o; p.lse = lse; p.raw_score = raw_score; p.raw_ld = raw_ld;
   p.score_head_as_written = score_head_as_written;
-  p.part = (float*)workspace; p.nsplit = dec_splits(max_keys); p.max_keys = (int)max_keys;
+  p.tile_prefix = (int32_t*)workspace; p.part = (float*)((char*)workspace + dec_ws_prefix_bytes(batch));
+  p.max_keys = (int)max_keys;
   int rc = dec_dispatch<DEC_MODE_COMPRESSED>(dtype, head_dim, p, (hipStream_t)stream_);
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_decode_cmpattn");
@@ -512,8 +612,7 @@ extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void
                 "fsa_decode_selattn: num_q_heads must be a multiple of num_kv_heads");
   FSA_CHECK_ARG(num_q_heads / num_kv_heads <= 16, "fsa_decode_selattn: at most 16 query heads per kv head");
   FSA_CHECK_ARG(batch >= 1 && topk >= 1 && block_size >= 1, "fsa_decode_selattn: bad sizes");
-  const int64_t max_keys = (int64_t)topk * ((block_size + DEC_TK - 1) / DEC_TK) * DEC_TK;
-  FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim, max_keys),
+  FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim),
                 "fsa_decode_selattn: workspace too small (see fsa_decode_workspace_bytes)");
   DecParams p = {};
   p.q = q; p.k = k_cache; p.v = v_cache; p.q_sb = q_stride_b; p.q_sh = q_stride_h;
@@ -521,7 +620,7 @@ extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void
   p.cu_k = cu_k; p.topk_idx = topk_idx; p.batch = batch; p.hq = num_q_heads; p.hkv = num_kv_heads;
   p.g = num_q_heads / num_kv_heads; p.topk = topk; p.block_size = block_size;
   p.scale_log2 = softmax_scale * LOG2E; p.o = o; p.lse = lse;
-  p.part = (float*)workspace; p.nsplit = dec_splits(max_keys);
+  p.tile_prefix = (int32_t*)workspace; p.part = (float*)((char*)workspace + dec_ws_prefix_bytes(batch));
   int rc = dec_dispatch<DEC_MODE_SELECTED>(dtype, head_dim, p, (hipStream_t)stream_);
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_decode_selattn");

@@ -240,13 +240,15 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
  * attend every cached key of the selected blocks (ids < 0, past the cache or
  * repeated are ignored).
  *
- * Both attention calls split the keys of a request over several work-groups
- * and merge their fp32 partials in a fixed order: the caller provides a
- * workspace of fsa_decode_workspace_bytes(..., max_keys) bytes, max_keys being
- * a host upper bound of the keys one request attends (compressed: the longest
- * visible compressed cache, keys beyond it are ignored; selected: topk *
- * block_size rounded up to 32-key tiles).  At most 15 (compressed) / 16
- * (selected) query heads per kv head.
+ * Both attention calls run a grid of single-wave work-groups that stays
+ * resident for the whole launch; the key tiles of all (request, kv head) pairs
+ * are dealt to the waves in equal contiguous shares, and the fp32 partials of
+ * a pair are merged in a fixed order.  The caller provides a workspace of
+ * fsa_decode_workspace_bytes(...) bytes (max_keys is kept for compatibility
+ * and does not change the size).  max_keys of fsa_decode_cmpattn is a host
+ * upper bound of the visible compressed cache of one request (keys beyond it
+ * are ignored).  At most 15 (compressed) / 16 (selected) query heads per kv
+ * head.
  * ---------------------------------------------------------------------- */
 size_t fsa_decode_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
                                   int32_t head_dim, int64_t max_keys);

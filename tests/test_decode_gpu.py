@@ -16,7 +16,7 @@ TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
 KS, ST = 32, 16
 
 
-def _caches(lens, hq, hkv, d, dtype, seed):
+def _caches(lens, hq, hkv, d, dtype, seed, raw=True):
     gen = torch.Generator().manual_seed(seed)
     b = len(lens)
     cu_k = [0]
@@ -26,8 +26,8 @@ def _caches(lens, hq, hkv, d, dtype, seed):
         cu_ck.append(cu_ck[-1] + ((l - KS) // ST + 1 if l >= KS else 0))
     std = 0.5 if d == 256 else 1.0
     q = (torch.randn(b, hq, d, generator=gen) * std).to(dtype)
-    kc = (torch.randn(cu_k[-1], hkv, d, generator=gen) * std).to(dtype)
-    vc = (torch.randn(cu_k[-1], hkv, d, generator=gen) * std).to(dtype)
+    kc = (torch.randn(cu_k[-1], hkv, d, generator=gen) * std).to(dtype) if raw else None
+    vc = (torch.randn(cu_k[-1], hkv, d, generator=gen) * std).to(dtype) if raw else None
     ck = (torch.randn(max(cu_ck[-1], 1), hkv, d, generator=gen) * std).to(dtype)
     cv = (torch.randn(max(cu_ck[-1], 1), hkv, d, generator=gen) * std).to(dtype)
     return q, kc, vc, ck, cv, cu_k, cu_ck
@@ -42,11 +42,23 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("lens,hq,hkv,d,bk,t,dtype", CASES)
+def _many_lens(n, lo, hi, seed):
+    gen = torch.Generator().manual_seed(seed)
+    return torch.randint(lo, hi + 1, (n,), generator=gen).tolist()
+
+
+# Many requests: the tile sequence is longer than the persistent grid, so a wave's share holds several tiles and
+# crosses (request, kv head) boundaries, requests without any compressed key included.
+MANY_COMPRESSED = (_many_lens(120, 16, 40000, 77), 8, 2, 128, 64, 16, torch.bfloat16)
+MANY_SELECTED = (_many_lens(300, 40, 1500, 78), 8, 2, 128, 64, 16, torch.bfloat16)
+
+
+@pytest.mark.parametrize("lens,hq,hkv,d,bk,t,dtype", CASES + [MANY_COMPRESSED])
 @pytest.mark.parametrize("as_written", [False, True])
 def test_decode_compressed_and_topk(dev, lens, hq, hkv, d, bk, t, dtype, as_written):
-    print(f"case lens={lens} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype} as_written={as_written}", flush=True)
-    q, kc, vc, ck, cv, cu_k, cu_ck = _caches(lens, hq, hkv, d, dtype, seed=21)
+    print(f"case lens={lens[:8]}{'...' if len(lens) > 8 else ''} ({len(lens)} requests) hq={hq} hkv={hkv} d={d} bk={bk} "
+          f"t={t} {dtype} as_written={as_written}", flush=True)
+    q, kc, vc, ck, cv, cu_k, cu_ck = _caches(lens, hq, hkv, d, dtype, seed=21, raw=False)
     pos = torch.tensor([l - 1 for l in lens], dtype=torch.int32)
     seqlens = torch.tensor(lens, dtype=torch.int32)
     max_ck = max(b_ - a_ for a_, b_ in zip(cu_ck[:-1], cu_ck[1:]))
@@ -82,9 +94,10 @@ def test_decode_compressed_and_topk(dev, lens, hq, hkv, d, bk, t, dtype, as_writ
     assert diff <= 2e-3
 
 
-@pytest.mark.parametrize("lens,hq,hkv,d,bk,t,dtype", CASES)
+@pytest.mark.parametrize("lens,hq,hkv,d,bk,t,dtype", CASES + [MANY_SELECTED])
 def test_decode_selected(dev, lens, hq, hkv, d, bk, t, dtype):
-    print(f"case lens={lens} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    print(f"case lens={lens[:8]}{'...' if len(lens) > 8 else ''} ({len(lens)} requests) hq={hq} hkv={hkv} d={d} bk={bk} "
+          f"t={t} {dtype}", flush=True)
     q, kc, vc, ck, cv, cu_k, cu_ck = _caches(lens, hq, hkv, d, dtype, seed=22)
     gen = torch.Generator().manual_seed(5)
     b = len(lens)
