@@ -243,7 +243,9 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
  * Both attention calls run a grid of single-wave work-groups that stays
  * resident for the whole launch; the key tiles of all (request, kv head) pairs
  * are dealt to the waves in equal contiguous shares, and the fp32 partials of
- * a pair are merged in a fixed order.  The caller provides a workspace of
+ * a pair are merged in a fixed order (results are reproducible for a given
+ * batch; across different batches a request's output agrees up to fp32
+ * rounding of the partial sums).  The caller provides a workspace of
  * fsa_decode_workspace_bytes(...) bytes (max_keys is kept for compatibility
  * and does not change the size).  max_keys of fsa_decode_cmpattn is a host
  * upper bound of the visible compressed cache of one request (keys beyond it
