@@ -563,8 +563,7 @@ cmp_topk_kernel(TopkParams p) {
       uint32_t best = key[0];
 #pragma unroll
       for (int r = 1; r < NREG; ++r) best = max(best, key[r]);
-#pragma unroll
-      for (int o = 32; o >= 1; o >>= 1) best = max(best, (uint32_t)__shfl_xor((int)best, o, 64));
+      best = wave_max_u32(best);
 #pragma unroll
       for (int r = 0; r < NREG; ++r) key[r] = key[r] == best ? 0u : key[r];  // keys are distinct
       if (lane == t) my_id = 0xFFFF - (int)(best & 0xFFFFu);
@@ -583,15 +582,11 @@ cmp_topk_kernel(TopkParams p) {
           best_id = b;
         }
       }
-#pragma unroll
-      for (int o = 32; o >= 1; o >>= 1) {
-        const float ov = __shfl_xor(best, o, 64);
-        const int oi = __shfl_xor(best_id, o, 64);
-        if (ov > best || (ov == best && oi < best_id)) {
-          best = ov;
-          best_id = oi;
-        }
-      }
+      // scores are >= 0 (or the -2 of a lane without blocks): as 64-bit keys, score bits above and the complement
+      // of the id below, the larger key is the larger score or, on equal scores, the lower id
+      const uint64_t mine = best < 0.f ? 0ull : ((uint64_t)__float_as_uint(best) << 32) | (0xFFFFFFFFu - (uint32_t)best_id);
+      const uint64_t top = wave_max_u64(mine);
+      best_id = (int)(0xFFFFFFFFu - (uint32_t)top);
       if (lane == t) my_id = best_id;
       if (lane == 0) bs[best_id] = -1.f;
       __builtin_amdgcn_wave_barrier();
@@ -601,7 +596,7 @@ cmp_topk_kernel(TopkParams p) {
   const int t_eff = min(p.t_out, 64);
   int rank = 0;
   for (int t = 0; t < t_eff; ++t) {
-    const int other = __shfl(my_id, t, 64);
+    const int other = __builtin_amdgcn_readlane(my_id, t);  // uniform lane index: no trip through the LDS crossbar
     if (other < my_id) ++rank;
   }
   if (lane < t_eff)

@@ -432,14 +432,13 @@ decode_topk_kernel(DecTopkParams p) {
         best_id = blk;
       }
     }
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) {
-      const float ov = __shfl_xor(best, o, 64);
-      const int oi = __shfl_xor(best_id, o, 64);
-      if (ov > best || (ov == best && oi < best_id)) {
-        best = ov;
-        best_id = oi;
-      }
+    {
+      // scores are >= 0 (negative: nothing left in this lane): as 64-bit keys, score bits above and the complement of
+      // the id below, the larger key is the larger score or, on equal scores, the lower id
+      const uint64_t mine = best < 0.f ? 0ull : ((uint64_t)__float_as_uint(best) << 32) | (0xFFFFFFFFu - (uint32_t)best_id);
+      const uint64_t top = wave_max_u64(mine);
+      best = top ? __uint_as_float((uint32_t)(top >> 32)) : -2.f;
+      best_id = top ? (int)(0xFFFFFFFFu - (uint32_t)top) : 0x7fffffff;
     }
     if (lane == 0) {
       wbest[wv] = best;

@@ -149,6 +149,38 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// Maximum of an unsigned value over the wave, returned to every lane, without going through the LDS crossbar:
+// prefix maxima inside each row of 16 lanes with the DPP row shifts (lanes shifted in from outside a row read 0),
+// the rows combined with the two DPP row broadcasts, the result read from the last lane.
+template <int CTRL, int ROW_MASK, bool ZERO_FILL> __device__ __forceinline__ uint32_t dpp_move(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, ROW_MASK, 0xf, ZERO_FILL);
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t x) {
+  x = max(x, dpp_move<0x111, 0xf, true>(x));   // row_shr:1
+  x = max(x, dpp_move<0x112, 0xf, true>(x));   // row_shr:2
+  x = max(x, dpp_move<0x114, 0xf, true>(x));   // row_shr:4
+  x = max(x, dpp_move<0x118, 0xf, true>(x));   // row_shr:8 -> lane 15 of a row holds the maximum of the row
+  x = max(x, dpp_move<0x142, 0xa, false>(x));  // row_bcast:15 into rows 1 and 3
+  x = max(x, dpp_move<0x143, 0xc, false>(x));  // row_bcast:31 into rows 2 and 3
+  return (uint32_t)__builtin_amdgcn_readlane((int)x, 63);
+}
+// the same for 64-bit keys (hi word compared first)
+template <int CTRL, int ROW_MASK, bool ZERO_FILL> __device__ __forceinline__ uint64_t dpp_max_u64(uint64_t x) {
+  const uint64_t y = ((uint64_t)dpp_move<CTRL, ROW_MASK, ZERO_FILL>((uint32_t)(x >> 32)) << 32) |
+                     dpp_move<CTRL, ROW_MASK, ZERO_FILL>((uint32_t)x);
+  return y > x ? y : x;
+}
+__device__ __forceinline__ uint64_t wave_max_u64(uint64_t x) {
+  x = dpp_max_u64<0x111, 0xf, true>(x);
+  x = dpp_max_u64<0x112, 0xf, true>(x);
+  x = dpp_max_u64<0x114, 0xf, true>(x);
+  x = dpp_max_u64<0x118, 0xf, true>(x);
+  x = dpp_max_u64<0x142, 0xa, false>(x);
+  x = dpp_max_u64<0x143, 0xc, false>(x);
+  return ((uint64_t)(uint32_t)__builtin_amdgcn_readlane((int)(x >> 32), 63) << 32) |
+         (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)x, 63);
+}
+
 // r / g for a row index r >= 0 and a GQA group of g heads: a shift where g is a power of two (g_shift =
 // log2 g), the division otherwise (g_shift < 0).  The general division costs some forty instructions and sits in
 // the address computation of every gathered row.
