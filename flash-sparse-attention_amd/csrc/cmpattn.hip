@@ -504,6 +504,7 @@ struct TopkParams {
   int64_t n_tokens;
   int hkv;
   int kernel_size, kernel_stride, block_size;
+  int na, ne;           // kernel_size / kernel_stride, block_size / kernel_stride
   int nblk;             // columns of the block-score matrix: ceil(max_seqlen_q / block_size)
   int t_out;            // min(topk, nblk)
   int init_blocks, local_blocks;
@@ -523,22 +524,41 @@ __global__ void __launch_bounds__(256)
 cmp_topk_kernel(TopkParams p) {
   extern __shared__ float bs_all[];  // [4 waves][nblk], NREG == 0 only
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int64_t row = (int64_t)blockIdx.x * 4 + wv;
-  if (row >= p.n_tokens * p.hkv) return;
-  const int h = (int)(row / p.n_tokens);
-  const int tok = (int)(row - (int64_t)h * p.n_tokens);
+  const int h = blockIdx.y;
+  const int tok = blockIdx.x * 4 + wv;  // the same for every lane of the wave
+  if (tok >= p.n_tokens) return;
   float* bs = bs_all + wv * p.nblk;
   const int s = upper_seg(p.cu_q, p.batch, tok);
   const int qi = tok - p.cu_q[s];
   const int nc = p.cu_k[s + 1] - p.cu_k[s];
   const int n_vis = qi >= p.kernel_size - 1 ? min(nc, (qi - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
-  const int na = p.kernel_size / p.kernel_stride, ne = p.block_size / p.kernel_stride;
+  const int na = p.na, ne = p.ne;
   const int n_off = na + ne - 1, pad = na - 1;
   const int bq = qi / p.block_size;
   const float* srow = p.score + ((int64_t)h * p.n_tokens + tok) * p.score_ld;
+  // the usual geometry (compression window of 2 strides, selection block of 4): taps 4 b - 1 .. 4 b + 3 with
+  // weights 1 2 2 2 1, four of them one aligned 16-byte load (score rows start 16-byte aligned)
+  const bool taps_12221 = na == 2 && ne == 4;
   auto block_score = [&](int b) {
     float acc = 0.f;
     const int c0 = b * ne - pad;
+    if (taps_12221) {
+      const int c = 4 * b;
+      f32x4 x = {0.f, 0.f, 0.f, 0.f};
+      if (c + 3 < n_vis) {
+        x = *reinterpret_cast<const f32x4*>(srow + c);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 3; ++e)
+          if (c + e < n_vis) x[e] = srow[c + e];
+      }
+      const float xm = (c >= 1 && c - 1 < n_vis) ? srow[c - 1] : 0.f;
+      acc = xm;
+      acc += 2.f * x[0];
+      acc += 2.f * x[1];
+      acc += 2.f * x[2];
+      acc += x[3];
+    } else
     for (int o = 0; o < n_off; ++o) {
       const int c = c0 + o;
       if (c >= 0 && c < n_vis) {
@@ -894,12 +914,12 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   tp.score = p.score; tp.score_ld = p.score_ld; tp.cu_q = cu_seqlens_q; tp.cu_k = cu_seqlens_k;
   tp.batch = batch; tp.n_tokens = total_q; tp.hkv = num_kv_heads;
   tp.kernel_size = kernel_size; tp.kernel_stride = kernel_stride; tp.block_size = block_size;
+  tp.na = kernel_size / kernel_stride; tp.ne = block_size / kernel_stride;
   tp.nblk = nblk; tp.t_out = t_out; tp.init_blocks = init_blocks; tp.local_blocks = local_blocks;
   tp.to_bf16 = scores_to_bf16; tp.topk_idx = topk_idx; tp.block_score = block_score;
   {
     ProfScope ps_("cmp_topk", stream);
-    const int64_t rows = total_q * num_kv_heads;
-    const unsigned grid = (unsigned)((rows + 3) / 4);
+    const dim3 grid((unsigned)((total_q + 3) / 4), (unsigned)num_kv_heads);
     if (scores_to_bf16 && nblk <= 128) cmp_topk_kernel<2><<<grid, 256, 0, stream>>>(tp);
     else if (scores_to_bf16 && nblk <= 256) cmp_topk_kernel<4><<<grid, 256, 0, stream>>>(tp);
     else if (scores_to_bf16 && nblk <= 512) cmp_topk_kernel<8><<<grid, 256, 0, stream>>>(tp);
