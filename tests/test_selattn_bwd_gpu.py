@@ -34,6 +34,12 @@ CASES = [
     ([0, 512], 4, 1, 64, 64, 16, torch.bfloat16, 1.0),
     ([0, 33], 2, 2, 128, 64, 16, torch.bfloat16, 1.0),
     ([0, 9000], 2, 1, 128, 64, 16, torch.bfloat16, 1.0),   # block 0 spans several dK/dV work-groups
+    # the remaining (head_dim, block size) pairs of the dispatch table
+    ([0, 900], 4, 2, 128, 128, 4, torch.bfloat16, 1.0),
+    ([0, 700], 4, 2, 64, 32, 6, torch.bfloat16, 1.0),
+    ([0, 900], 2, 2, 64, 128, 4, torch.float16, 1.0),
+    ([0, 500], 4, 2, 256, 32, 6, torch.float16, 0.5),
+    ([0, 700], 2, 1, 256, 64, 6, torch.bfloat16, 0.5),
 ]
 
 
