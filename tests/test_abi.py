@@ -59,3 +59,24 @@ def test_wrappers_refuse_cpu_tensors():
     t = torch.zeros(1, 4, 2, dtype=torch.int32)
     with pytest.raises(RuntimeError, match="no CPU path"):
         ops.build_index(t, torch.tensor([0, 4], dtype=torch.int32), 64)
+
+
+def test_every_compute_entry_point_rejects_null_pointers():
+    """All-zero arguments: each entry point must answer with the invalid-argument code and a message before it
+    touches a device (this runs on machines without a GPU)."""
+    lib = _lib.load()
+    skip = {"fsa_version", "fsa_profile_enable", "fsa_profile_count"}
+    for name, (res, args) in _lib.SIGNATURES.items():
+        if res is not C.c_int or name in skip:
+            continue
+        vals = []
+        for a in args:
+            if a in (C.c_void_p, C.c_char_p) or getattr(a, "__name__", "").startswith("LP_"):
+                vals.append(None)
+            elif a in (C.c_float, C.c_double):
+                vals.append(0.0)
+            else:
+                vals.append(0)
+        rc = getattr(lib, name)(*vals)
+        assert rc == -1, (name, rc)
+        assert lib.fsa_last_error(), name
