@@ -1,0 +1,86 @@
+"""GPU parity over drawn configurations: ragged batches, GQA groups 1..8 (3 and 6 included), head dims 64 / 128,
+block sizes 32 / 64 / 128, top-k 3..16, block lists in arbitrary slot order with padding anywhere.
+
+Same bars as the fixed cases: index lists bit-exact, O max-abs 2e-2 (bf16) / 5e-3 (fp16), base-2 LSE 1e-3,
+gradients within the same bound plus one ulp of the output dtype.
+"""
+import numpy as np
+import pytest
+import torch
+
+from fsa_hip import ops
+from fsa_hip.synth import make_qkv, make_topk_idx
+from oracle import selattn as orc
+
+pytestmark = pytest.mark.gpu
+
+O_TOL = {torch.bfloat16: 2e-2, torch.float16: 5e-3}
+ULP = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}
+
+
+def _draw(seed):
+    rng = np.random.default_rng(seed)
+    nseq = int(rng.integers(1, 5))
+    lens = [int(rng.choice([1, 7, 63, 64, 65, 200, 777, 1500, 2600])) for _ in range(nseq)]
+    if seed % 4 == 0:
+        lens[0] = 3100                     # block 0 of this sequence is shared by several dK/dV work-groups
+    cu = [0]
+    for l in lens:
+        cu.append(cu[-1] + l)
+    hkv = int(rng.choice([1, 2, 3]))
+    g = int(rng.choice([1, 2, 3, 4, 6, 8]))
+    d = int(rng.choice([64, 128]))
+    bk = int(rng.choice([32, 64, 128]))
+    t = int(rng.choice([3, 5, 8, 16]))
+    dtype = torch.bfloat16 if rng.integers(2) else torch.float16
+    return cu, hkv * g, hkv, d, bk, t, dtype
+
+
+def _scramble(topk, seed):
+    """Slots of every query in a random order, and one in eight non-forced entries replaced by padding."""
+    gen = torch.Generator().manual_seed(seed)
+    hkv, n, t = topk.shape
+    drop = (torch.rand(hkv, n, t, generator=gen) < 0.125) & (topk > 0)
+    out = torch.where(drop, torch.full_like(topk, -1), topk)
+    perm = torch.rand(hkv, n, t, generator=gen).argsort(-1)
+    return torch.gather(out, 2, perm).contiguous()
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_drawn_configuration(dev, seed):
+    cu, hq, hkv, d, bk, t, dtype = _draw(seed)
+    print(f"case seed={seed} cu={cu} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    n = cu[-1]
+    std = 1.0 if dtype == torch.bfloat16 else 0.5
+    q, k, v, do = make_qkv(n, hq, hkv, d, dtype, seed=100 + seed, std=std)
+    topk = _scramble(make_topk_idx(cu, hkv, bk, t, seed=200 + seed), 300 + seed)
+    cu_t = torch.tensor(cu, dtype=torch.int32)
+    index = ops.build_index(topk.to(dev), cu_t.to(dev), bk)
+    cu_blocks, counts, starts, sel_tokens, slot_of = orc.build_index_ref(topk, cu, bk)
+    nb = int(cu_blocks[-1])
+    assert np.array_equal(index.counts.cpu().numpy()[:, :nb], counts)
+    assert np.array_equal(index.starts.cpu().numpy()[:, : nb + 1], starts)
+    assert np.array_equal(index.sel_tokens.cpu().numpy(), sel_tokens)
+    assert np.array_equal(index.slot_of.cpu().numpy(), slot_of)
+
+    qd, kd, vd, dod = (x.to(dev) for x in (q, k, v, do))
+    o, lse = ops.selattn_fwd(qd, kd, vd, index)
+    dq, dk, dv = ops.selattn_bwd(qd, kd, vd, o, dod, lse, index)
+    torch.cuda.synchronize()
+    o_ref, lse_ref = orc.selected_attention_ref(q.float(), k.float(), v.float(), topk, bk, cu)
+    lse_c = lse.cpu()
+    dead = torch.isinf(lse_ref)
+    assert torch.equal(torch.isinf(lse_c), dead)
+    err_o = (o.float().cpu() - o_ref).abs().max().item()
+    err_l = (lse_c[~dead] - lse_ref[~dead]).abs().max().item() if (~dead).any() else 0.0
+    print(f"  max|dO|={err_o:.3e} max|dLSE|={err_l:.3e}", flush=True)
+    assert err_o <= O_TOL[dtype] and err_l <= 1e-3
+    _, _, dq_r, dk_r, dv_r = orc.selected_attention_grads_ref(q.float(), k.float(), v.float(), topk, bk, cu,
+                                                              do.float(), round_dtype=dtype,
+                                                              o_in=o.float().cpu(), lse_in=lse_c)
+    for name, got, ref in (("dq", dq, dq_r), ("dk", dk, dk_r), ("dv", dv, dv_r)):
+        got = got.float().cpu()
+        assert torch.isfinite(got).all(), name
+        excess = ((got - ref).abs() - ULP[dtype] * ref.abs()).max().item()
+        print(f"  max|d{name}|={(got - ref).abs().max().item():.3e}", flush=True)
+        assert excess <= O_TOL[dtype], name
