@@ -30,6 +30,10 @@ CASES = [
     ([0, 1500], 6, 2, 64, 32, 16, 64, 8, torch.float16),                       # g = 3
     ([0, 1024], 4, 2, 256, 32, 16, 128, 8, torch.float16),
     ([0, 4096], 16, 4, 128, 32, 16, 64, 16, torch.bfloat16),
+    # other window / stride / block geometries (tap weights of the re-binning other than 1 2 2 2 1)
+    ([0, 1800], 4, 2, 128, 64, 16, 64, 8, torch.bfloat16),
+    ([0, 1300, 2000], 4, 2, 128, 16, 16, 32, 6, torch.float16),
+    ([0, 1500], 2, 1, 64, 32, 8, 64, 8, torch.bfloat16),
 ]
 
 
