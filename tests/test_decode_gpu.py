@@ -126,3 +126,15 @@ def test_decode_selected(dev, lens, hq, hkv, d, bk, t, dtype):
     o_wr, lse_wr = orc.as_written_selected_ref(q.float(), kc.float(), vc.float(), cu_k)
     assert (o_w.float().cpu() - o_wr).abs().max().item() <= 1e-6
     assert (lse_w.cpu() - lse_wr).abs().max().item() <= 1e-3
+
+
+@pytest.mark.parametrize("ks,st,bk", [(64, 16, 64), (16, 16, 32), (32, 8, 64)])
+def test_decode_other_geometries(dev, monkeypatch, ks, st, bk):
+    """Compression windows / strides / block sizes other than 32 / 16 / 64 (other tap weights of the re-binning)."""
+    import sys
+    me = sys.modules[__name__]
+    monkeypatch.setattr(me, "KS", ks)
+    monkeypatch.setattr(me, "ST", st)
+    lens = [3000, 100, ks - 1, 1700]
+    test_decode_compressed_and_topk(dev, lens, 8, 2, 128, bk, 8, torch.bfloat16, False)
+    test_decode_selected(dev, lens, 8, 2, 128, bk, 8, torch.bfloat16)
