@@ -538,18 +538,18 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 
 // Blocks with no selecting query get zeros; blocks split over several
 // work-groups get the fixed-order sum of their fp32 partials.
-template <typename T, int D, int BK, int MODE>
-__global__ void __launch_bounds__(256)
-attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
+// (bx, h, bz) of n_z: the position of the work-group in the grid of attn_bwd_dkdv_reduce_kernel; UB partial loads
+// are issued together
+template <typename T, int D, int BK, int MODE, int UB>
+__device__ __forceinline__ void dkdv_reduce_block(const SelBwdParams& p, int bx, int h, int bz, int n_z) {
   typedef typename Elem<T>::vec4 vec4;
-  const int h = blockIdx.y;
   const int32_t* tp = p.tile_prefix + h * (p.max_blocks + 1);
   const int n_blocks = p.cu_blocks[p.batch];
   // a work-group looks at KV_REDUCE_SPAN blocks at once: almost all of them have a single tile, whose
   // work-group wrote dK / dV itself
   __shared__ int todo[KV_REDUCE_SPAN];
   __shared__ int n_todo;
-  const int gb0 = blockIdx.x * KV_REDUCE_SPAN;
+  const int gb0 = bx * KV_REDUCE_SPAN;
   if (threadIdx.x < WAVE) {
     static_assert(KV_REDUCE_SPAN == WAVE, "one lane per block of the span");
     const int gbi = gb0 + threadIdx.x;
@@ -562,7 +562,7 @@ attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
   // unit of work: 256 consecutive (key, 4 dims) items of one block; the gridDim.z work-groups of the span
   // take the units round-robin
   constexpr int CH = BK * (D / 4) / 256;
-  for (int u_ = blockIdx.z; u_ < n_todo * CH; u_ += gridDim.z) {
+  for (int u_ = bz; u_ < n_todo * CH; u_ += n_z) {
     const int gb = todo[u_ / CH];
     const int t0 = tp[gb], nt = tp[gb + 1] - t0;
     KvBlock<MODE, BK> blk;
@@ -575,7 +575,6 @@ attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
       f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = {0.f, 0.f, 0.f, 0.f};
       const float* part0 = p.dkdv_part + ((int64_t)h * p.max_tiles + t0) * (2 * BK * D) + key * D + d4;
       // the loads of a batch are issued together (one memory latency per batch), the adds keep the tile order
-      constexpr int UB = 8;
       for (int tb = 0; tb < nt; tb += UB) {
         f32x4 xk[UB], xv[UB];
 #pragma unroll
@@ -601,6 +600,12 @@ attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
       store8(reinterpret_cast<T*>(p.dv) + (int64_t)tok * p.dk_sn + (int64_t)h * p.dk_sh + d4, b);
     }
   }
+}
+
+template <typename T, int D, int BK, int MODE>
+__global__ void __launch_bounds__(256)
+attn_bwd_dkdv_reduce_kernel(SelBwdParams p) {
+  dkdv_reduce_block<T, D, BK, MODE, 8>(p, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z);
 }
 
 

@@ -181,14 +181,13 @@ selattn_bwd_dq_kernel(SelBwdParams p) {
 
 // Sum of the <= T partial dQ rows of each (query, head); undoes the lane-native order.
 template <typename T, int D>
-__global__ void __launch_bounds__(256)
-selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __restrict__ slot_of,
-                             int64_t cap, int64_t n_tokens, int hq, int g, int topk, int natural,
-                             T* __restrict__ dq /* contiguous [N, Hq, D] */) {
+__device__ __forceinline__ void dq_reduce_block(const T* __restrict__ dq_part, const int32_t* __restrict__ slot_of,
+                                                int64_t cap, int64_t n_tokens, int hq, int g, int topk, int natural,
+                                                T* __restrict__ dq /* contiguous [N, Hq, D] */, int64_t block) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
   constexpr int LPR = D / 8, RPB = 256 / LPR;
-  const int64_t R = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+  const int64_t R = block * RPB + threadIdx.x / LPR;
   const int sub = threadIdx.x % LPR;
   if (R >= n_tokens * hq) return;
   const int64_t tok = R / hq;
@@ -234,6 +233,37 @@ selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __res
   store8(orow + 8, b);
 }
 
+template <typename T, int D>
+__global__ void __launch_bounds__(256)
+selattn_bwd_dq_reduce_kernel(const T* __restrict__ dq_part, const int32_t* __restrict__ slot_of,
+                             int64_t cap, int64_t n_tokens, int hq, int g, int topk, int natural,
+                             T* __restrict__ dq) {
+  dq_reduce_block<T, D>(dq_part, slot_of, cap, n_tokens, hq, g, topk, natural, dq, blockIdx.x);
+}
+
+// The two reductions that end the fused backward in one launch: the first n_kv work-groups add up the fp32 dK / dV
+// partials of the blocks that were shared by several work-groups (few, and latency bound), the others the partial
+// dQ rows, so the small reduction runs in the shadow of the large one instead of after it.
+struct DqReduceArgs {
+  const void* dq_part;
+  const int32_t* slot_of;
+  int64_t cap, n_tokens;
+  int hq, g, topk;
+  void* dq;
+};
+template <typename T, int D, int BK>
+__global__ void __launch_bounds__(256)
+selattn_bwd_reduce_kernel(SelBwdParams p, DqReduceArgs a, int n_kv, int hkv) {
+  const int b = blockIdx.x;
+  if (b < n_kv) {
+    const int bz = b % KV_REDUCE_SPLIT, h = (b / KV_REDUCE_SPLIT) % hkv, bx = b / (KV_REDUCE_SPLIT * hkv);
+    dkdv_reduce_block<T, D, BK, KV_MODE_SELECTED, 4>(p, bx, h, bz, KV_REDUCE_SPLIT);
+  } else {
+    dq_reduce_block<T, D>((const T*)a.dq_part, a.slot_of, a.cap, a.n_tokens, a.hq, a.g, a.topk, 1, (T*)a.dq,
+                          (int64_t)(b - n_kv));
+  }
+}
+
 // ------------------------------------------------------------- host side ----
 struct BwdWs {
   size_t off_delta, off_dqpart, off_tiles_dq, off_tiles_kv, off_kvpart, total;
@@ -277,40 +307,48 @@ template <typename K> static int set_lds(K kernel, int bytes) {
 
 template <typename T, int D, int BK>
 static int launch_bwd(const SelBwdParams& pdq, const SelBwdParams& pkv, int hkv, int64_t tiles_dq,
-                      int64_t tiles_kv, hipStream_t stream) {
+                      int64_t tiles_kv, const DqReduceArgs& red, hipStream_t stream) {
   int rc = 0;
+  const unsigned kv_spans = (unsigned)((pkv.max_blocks + KV_REDUCE_SPAN - 1) / KV_REDUCE_SPAN);
   if (fused_dq()) {
     rc = set_lds(attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED, true>, KvCfg<D, BK>::BYTES_FUSED);
     if (rc) return rc;
-    ProfScope ps_("selattn_bwd_dqdkdv", stream);
-    attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED, true>
-        <<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES_FUSED, stream>>>(pkv);
-  } else {
-    rc = set_lds(selattn_bwd_dq_kernel<T, D, BK>, DqLds<D, BK>::BYTES);
-    if (rc) return rc;
-    rc = set_lds(attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED>, KvCfg<D, BK>::BYTES);
-    if (rc) return rc;
     {
-      ProfScope ps_("selattn_bwd_dq", stream);
-      selattn_bwd_dq_kernel<T, D, BK><<<dim3((unsigned)tiles_dq, hkv), DQ_THREADS, DqLds<D, BK>::BYTES, stream>>>(pdq);
+      ProfScope ps_("selattn_bwd_dqdkdv", stream);
+      attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED, true>
+          <<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES_FUSED, stream>>>(pkv);
     }
-    {
-      ProfScope ps_("selattn_bwd_dkdv", stream);
-      attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES, stream>>>(pkv);
-    }
+    constexpr int RPB = 256 / (D / 8);
+    const int64_t rows = red.n_tokens * red.hq;
+    const int64_t n_kv = (int64_t)kv_spans * hkv * KV_REDUCE_SPLIT, n_dq = (rows + RPB - 1) / RPB;
+    ProfScope ps_("selattn_bwd_dq_reduce", stream);
+    selattn_bwd_reduce_kernel<T, D, BK><<<(unsigned)(n_kv + n_dq), 256, 0, stream>>>(pkv, red, (int)n_kv, hkv);
+    return 0;
+  }
+  rc = set_lds(selattn_bwd_dq_kernel<T, D, BK>, DqLds<D, BK>::BYTES);
+  if (rc) return rc;
+  rc = set_lds(attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED>, KvCfg<D, BK>::BYTES);
+  if (rc) return rc;
+  {
+    ProfScope ps_("selattn_bwd_dq", stream);
+    selattn_bwd_dq_kernel<T, D, BK><<<dim3((unsigned)tiles_dq, hkv), DQ_THREADS, DqLds<D, BK>::BYTES, stream>>>(pdq);
+  }
+  {
+    ProfScope ps_("selattn_bwd_dkdv", stream);
+    attn_bwd_dkdv_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3((unsigned)tiles_kv, hkv), KvCfg<D, BK>::NT, KvCfg<D, BK>::BYTES, stream>>>(pkv);
   }
   {
     ProfScope ps_("selattn_bwd_dkdv_reduce", stream);
-    attn_bwd_dkdv_reduce_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3((unsigned)((pkv.max_blocks + KV_REDUCE_SPAN - 1) / KV_REDUCE_SPAN), hkv, KV_REDUCE_SPLIT), 256, 0, stream>>>(pkv);
+    attn_bwd_dkdv_reduce_kernel<T, D, BK, KV_MODE_SELECTED><<<dim3(kv_spans, hkv, KV_REDUCE_SPLIT), 256, 0, stream>>>(pkv);
   }
   return 0;
 }
 
 template <typename T>
 static int dispatch_bwd(int d, int bk, const SelBwdParams& pdq, const SelBwdParams& pkv, int hkv,
-                        int64_t tiles_dq, int64_t tiles_kv, hipStream_t stream) {
+                        int64_t tiles_dq, int64_t tiles_kv, const DqReduceArgs& red, hipStream_t stream) {
 #define FSA_CASE(DD, BB) \
-  if (d == DD && bk == BB) return launch_bwd<T, DD, BB>(pdq, pkv, hkv, tiles_dq, tiles_kv, stream);
+  if (d == DD && bk == BB) return launch_bwd<T, DD, BB>(pdq, pkv, hkv, tiles_dq, tiles_kv, red, stream);
   FSA_CASE(128, 64)
   FSA_CASE(128, 32)
   FSA_CASE(128, 128)
@@ -399,8 +437,11 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   float* delta = (float*)(wsp + ws.off_delta);
   int32_t* tiles_dq = (int32_t*)(wsp + ws.off_tiles_dq);
   int32_t* tiles_kv = (int32_t*)(wsp + ws.off_tiles_kv);
-  int rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, DQ_TILE_ROWS, tiles_dq, stream_);
-  if (rc) return rc;
+  int rc = 0;
+  if (!fused_dq()) {  // the tile list of the separate dQ kernel
+    rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, DQ_TILE_ROWS, tiles_dq, stream_);
+    if (rc) return rc;
+  }
   rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, kv_tile_rows(g, head_dim, block_size), tiles_kv, stream_);
   if (rc) return rc;
 
@@ -432,19 +473,24 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   pdq.tile_prefix = tiles_dq; pdq.max_tiles = ws.max_tiles_dq; pdq.kv_tile_rows = 0;
   pkv.tile_prefix = tiles_kv; pkv.max_tiles = ws.max_tiles_kv; pkv.kv_tile_rows = kv_tile_rows(g, head_dim, block_size);
 
+  DqReduceArgs red;
+  red.dq_part = p.dq_part; red.slot_of = slot_of; red.cap = cap; red.n_tokens = total_tokens;
+  red.hq = num_q_heads; red.g = g; red.topk = topk; red.dq = dq;
   rc = dtype == FSA_BF16
            ? dispatch_bwd<__bf16>(head_dim, block_size, pdq, pkv, num_kv_heads, ws.max_tiles_dq,
-                                  ws.max_tiles_kv, stream)
+                                  ws.max_tiles_kv, red, stream)
            : dispatch_bwd<_Float16>(head_dim, block_size, pdq, pkv, num_kv_heads, ws.max_tiles_dq,
-                                    ws.max_tiles_kv, stream);
+                                    ws.max_tiles_kv, red, stream);
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_selattn_bwd dq/dkdv");
-  rc = dtype == FSA_BF16
-           ? launch_rowwise<__bf16>(head_dim, nullptr, 0, 0, nullptr, 0, 0, total_tokens, num_q_heads,
-                                    nullptr, p.dq_part, slot_of, cap, g, topk, dq, true, stream)
-           : launch_rowwise<_Float16>(head_dim, nullptr, 0, 0, nullptr, 0, 0, total_tokens, num_q_heads,
-                                      nullptr, p.dq_part, slot_of, cap, g, topk, dq, true, stream);
-  if (rc) return rc;
+  if (!fused_dq()) {  // the fused path ends with the combined reduction launched above
+    rc = dtype == FSA_BF16
+             ? launch_rowwise<__bf16>(head_dim, nullptr, 0, 0, nullptr, 0, 0, total_tokens, num_q_heads,
+                                      nullptr, p.dq_part, slot_of, cap, g, topk, dq, true, stream)
+             : launch_rowwise<_Float16>(head_dim, nullptr, 0, 0, nullptr, 0, 0, total_tokens, num_q_heads,
+                                        nullptr, p.dq_part, slot_of, cap, g, topk, dq, true, stream);
+    if (rc) return rc;
+  }
   FSA_CHECK_LAUNCH("fsa_selattn_bwd dq reduce");
   return 0;
 }
