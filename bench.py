@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 # (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by the factor that makes the same counter
 # read 1 GiB for the 1 GiB device copy of --calib-copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
 PMC_TRAFFIC_BYTES = {
-    ("selattn_bwd_dqdkdv", 4): 13548389376,
+    ("selattn_bwd_dqdkdv", 4): 13549486080,
     ("selattn_bwd_dqdkdv", 2): 6610281472,
     ("selattn_bwd_dqdkdv", 1): 3254586368,
     ("selattn_fwd_main", 4): 8274831360,
