@@ -15,34 +15,53 @@
 namespace fsa {
 
 // ------------------------------------------------------------------- rope ----
-// One thread owns 8 + 8 dims (sub, sub + d/2) of one token for all heads: the angles depend on the position and
-// the dim only, so cos / sin are evaluated once per token instead of once per head.
-template <typename T>
+// One wave per token.  d/16 lanes cover a head (each lane 8 dims of the first half and their partners in the second
+// half), so a load instruction of the wave covers the half-rows of 64 / (d/16) neighbouring heads: the token's row
+// is read and written in contiguous 2*d-byte pieces.  The angles depend on the position and the dim only; every lane
+// evaluates the cos / sin of its 8 dims once and reuses them for all the heads it visits.  For the usual head dims
+// (LPR = d/16 a compile-time power of two) the lanes that share the same dims split the eight evaluations among
+// themselves and exchange the results, so a lane evaluates one or two angles instead of eight.
+template <typename T, int LPR>
 __global__ void __launch_bounds__(256)
 rope_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, T* __restrict__ out, int64_t o_sn,
             int64_t o_sh, const int32_t* __restrict__ cu, int batch, int64_t n, int h, int d,
             const float* __restrict__ inv_freq, float attn_scale, int start, int stride, int conj) {
   typedef typename Elem<T>::vec8 vec8;
-  const int lpr = d / 16;
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  const int64_t tok = idx / lpr;
-  const int sub = (int)(idx - tok * lpr);
+  const int lpr = LPR > 0 ? LPR : d / 16, hpw = WAVE / lpr;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int64_t tok = (int64_t)blockIdx.x * (256 / WAVE) + (threadIdx.x / WAVE);
   if (tok >= n) return;
+  const int sub = lane % lpr, hl = lane / lpr;
+  if (hl >= hpw) return;  // lanes left over where d/16 does not divide the wave
   const int s = upper_seg(cu, batch, (int)tok);
   const float pos = (float)(start + ((int)tok - cu[s]) * stride);
-  float c[8], sn[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float ang = pos * inv_freq[sub * 8 + e];
+  // the tables are rounded to the tensor's dtype before use, as in the reference
+  auto table = [&](int e, float& cv_out, float& sv_out) {
     float sv, cv;
-    sincosf(ang, &sv, &cv);
-    // the tables are rounded to the tensor's dtype before use, as in the reference
-    c[e] = (float)(T)(cv * attn_scale);
-    sn[e] = (float)(T)(sv * attn_scale);
-    if (conj) sn[e] = -sn[e];
+    sincosf(pos * inv_freq[sub * 8 + e], &sv, &cv);
+    cv_out = (float)(T)(cv * attn_scale);
+    sv_out = (float)(T)(sv * attn_scale);
+    if (conj) sv_out = -sv_out;
+  };
+  float c[8], sn[8];
+  if constexpr (LPR > 0) {
+    constexpr int HPW = WAVE / LPR;                  // lanes that hold the same dims
+    constexpr int PER = HPW >= 8 ? 1 : 8 / HPW;      // evaluations per lane
+    float cl[PER], sl[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) table((hl + i * HPW) % 8, cl[i], sl[i]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {  // dim e was evaluated by the lane with hl = e % HPW in its turn e / HPW
+      const int src = (e % HPW) * LPR + sub;
+      c[e] = __shfl(cl[HPW >= 8 ? 0 : e / HPW], src, WAVE);
+      sn[e] = __shfl(sl[HPW >= 8 ? 0 : e / HPW], src, WAVE);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) table(e, c[e], sn[e]);
   }
 #pragma unroll 4
-  for (int head = 0; head < h; ++head) {
+  for (int head = hl; head < h; head += hpw) {
     const T* xr = x + tok * x_sn + (int64_t)head * x_sh + sub * 8;
     vec8 a = load16<vec8>(xr), b = load16<vec8>(xr + d / 2);
     vec8 oa, ob;
@@ -447,22 +466,28 @@ extern "C" int fsa_rope(const void* x, void* out, int32_t dtype, int64_t x_strid
   hipStream_t stream = (hipStream_t)stream_;
   FSA_CHECK_ARG(x && out && cu_seqlens && inv_freq, "fsa_rope: null pointer");
   FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_rope: dtype must be bf16 or fp16");
-  FSA_CHECK_ARG(head_dim >= 16 && head_dim % 16 == 0, "fsa_rope: head_dim must be a multiple of 16");
+  FSA_CHECK_ARG(head_dim >= 16 && head_dim % 16 == 0 && head_dim <= 1024,
+                "fsa_rope: head_dim must be a multiple of 16, at most 1024");
   FSA_CHECK_ARG(batch >= 1 && num_heads >= 1, "fsa_rope: bad sizes");
   if (total_tokens == 0) return 0;
-  const int64_t work = total_tokens * (head_dim / 16);
-  const unsigned grid = (unsigned)((work + 255) / 256);
+  const unsigned grid = (unsigned)((total_tokens + 3) / 4);  // one wave per token
   ProfScope ps_("rope", stream);
-  if (dtype == FSA_BF16)
-    rope_kernel<__bf16><<<grid, 256, 0, stream>>>((const __bf16*)x, x_stride_n, x_stride_h, (__bf16*)out,
-                                                  o_stride_n, o_stride_h, cu_seqlens, batch, total_tokens,
-                                                  num_heads, head_dim, inv_freq, attention_scaling, start,
-                                                  stride, inverse);
-  else
-    rope_kernel<_Float16><<<grid, 256, 0, stream>>>((const _Float16*)x, x_stride_n, x_stride_h, (_Float16*)out,
-                                                    o_stride_n, o_stride_h, cu_seqlens, batch, total_tokens,
-                                                    num_heads, head_dim, inv_freq, attention_scaling, start,
-                                                    stride, inverse);
+#define FSA_ROPE(TT, LPR)                                                                                      \
+  rope_kernel<TT, LPR><<<grid, 256, 0, stream>>>((const TT*)x, x_stride_n, x_stride_h, (TT*)out, o_stride_n,   \
+                                                 o_stride_h, cu_seqlens, batch, total_tokens, num_heads,      \
+                                                 head_dim, inv_freq, attention_scaling, start, stride, inverse)
+#define FSA_ROPE_D(TT)                      \
+  if (head_dim == 64) FSA_ROPE(TT, 4);      \
+  else if (head_dim == 128) FSA_ROPE(TT, 8);  \
+  else if (head_dim == 256) FSA_ROPE(TT, 16); \
+  else FSA_ROPE(TT, 0)
+  if (dtype == FSA_BF16) {
+    FSA_ROPE_D(__bf16);
+  } else {
+    FSA_ROPE_D(_Float16);
+  }
+#undef FSA_ROPE_D
+#undef FSA_ROPE
   FSA_CHECK_LAUNCH("fsa_rope");
   return 0;
 }

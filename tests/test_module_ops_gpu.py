@@ -13,11 +13,12 @@ pytestmark = pytest.mark.gpu
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("start,stride", [(0, 1), (0, 16)])
-def test_rope(dev, dtype, start, stride):
+@pytest.mark.parametrize("h,d", [(6, 128), (32, 128), (3, 64), (5, 256), (4, 96)])
+def test_rope(dev, dtype, start, stride, h, d):
     gen = torch.Generator().manual_seed(41)
     cu = [0, 1000, 1001, 3000]
-    x = torch.randn(3000, 6, 128, generator=gen).to(dtype)
-    inv = orc.llama3_inv_freq(128, 500000.0)
+    x = torch.randn(3000, h, d, generator=gen).to(dtype)
+    inv = orc.llama3_inv_freq(d, 500000.0)
     cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
     y = ops.rope(x.to(dev), cu_t, inv.to(dev), 1.0, start, stride)
     back = ops.rope(y, cu_t, inv.to(dev), 1.0, start, stride, inverse=True)
