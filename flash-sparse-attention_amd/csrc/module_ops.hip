@@ -307,6 +307,13 @@ lc_dpe_kernel(const T* __restrict__ w, const float* __restrict__ dbias, T* __res
 }
 
 // dW[h, k, d, dout] = sum_n x[tok(n) + k, h, d] dY[n, h, dout] (+ pe[h,k,d] dbias[h,dout])
+// One work-group per (offset k, head, 128 input dims): few work-groups, each a long loop over all compressed
+// tokens, so a step covers many tokens (LCW_KC) to keep enough rows in flight.  (Cutting the output dims over more
+// work-groups was measured and is slower: the strided X rows, 256 bytes every kernel_stride tokens, are what the
+// kernel waits for, and every cut reads them again.)
+constexpr int LCW_KC = 128;
+template <int D> struct LcDwLds { static constexpr int BYTES = LCW_KC * ((128 + 16) + (D + 16)) * 2; };
+
 template <typename T, int D>
 __global__ void __launch_bounds__(256)
 lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __restrict__ dy,
@@ -314,10 +321,15 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
              const int32_t* __restrict__ cu_x, const int32_t* __restrict__ cu_y, int batch, int nheads,
              int ks, int stride) {
   typedef typename Elem<T>::vec8 vec8;
-  constexpr int XS = 128 + 16, YS = D + 16, NT = D / 32;  // 32 B pads: conflict-free transposing reads
-  __shared__ __attribute__((aligned(16))) T Xs[LC_KC * XS];
-  __shared__ __attribute__((aligned(16))) T Ys[LC_KC * YS];
-  const int k = blockIdx.x, h = blockIdx.y, dz = blockIdx.z * 128;
+  constexpr int LCW_DOUT = D;  // output dims per work-group
+  constexpr int XS = 128 + 16, YS = LCW_DOUT + 16, NT = LCW_DOUT / 32;  // 32 B pads: conflict-free transposing reads
+  constexpr int LC_KC = LCW_KC;  // compressed tokens per step of this kernel
+  constexpr int YC = LCW_DOUT / 8;  // 16-byte chunks of a dY row slice
+  extern __shared__ __attribute__((aligned(16))) unsigned char lcw_smem[];
+  T* Xs = reinterpret_cast<T*>(lcw_smem);
+  T* Ys = Xs + LC_KC * XS;
+  const int k = blockIdx.x, h = blockIdx.y;
+  const int dz = (blockIdx.z / (D / LCW_DOUT)) * 128, dout0 = (blockIdx.z % (D / LCW_DOUT)) * LCW_DOUT;
   const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
   const int col = lane & 31, hh = lane >> 5;
   const int ny_total = cu_y[batch];
@@ -328,28 +340,40 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
   // the rows of the next step travel while the current one is multiplied
-  constexpr int NX = LC_KC * 16 / 256, NY = LC_KC * (D / 8) / 256;
+  constexpr int NX = LC_KC * 16 / 256, NY = LC_KC * YC / 256;
+  static_assert(LC_KC * YC % 256 == 0, "dY slice must divide over the threads");
   vec8 xr[NX], yr[NY];
+  // token of compressed row n at window offset k (-1 past the end); found one step before the rows are requested,
+  // so that the search through cu_y is not part of the latency of a step
+  int64_t tok_of[NX];
+  auto find_tokens = [&](int n0) {
+#pragma unroll
+    for (int j = 0; j < NX; ++j) {
+      const int n = n0 + (tid + 256 * j) / 16;
+      tok_of[j] = -1;
+      if (n < ny_total) {
+        const int s = upper_seg(cu_y, batch, n);
+        tok_of[j] = cu_x[s] + (int64_t)(n - cu_y[s]) * stride + k;
+      }
+    }
+  };
   auto load_step = [&](int n0) {
 #pragma unroll
     for (int j = 0; j < NX; ++j) {  // X rows: 128 dims = 16 chunks
-      const int c = tid + 256 * j, r = c / 16, cc = c % 16;
-      const int n = n0 + r;
+      const int cc = (tid + 256 * j) % 16;
       xr[j] = zero8<T>();
-      if (n < ny_total) {
-        const int s = upper_seg(cu_y, batch, n);
-        const int64_t tok = cu_x[s] + (int64_t)(n - cu_y[s]) * stride + k;
-        xr[j] = load16<vec8>(x + tok * x_sn + (int64_t)h * x_sh + dz + cc * 8);
-      }
+      if (tok_of[j] >= 0) xr[j] = load16<vec8>(x + tok_of[j] * x_sn + (int64_t)h * x_sh + dz + cc * 8);
     }
+    find_tokens(n0 + LC_KC);
 #pragma unroll
     for (int j = 0; j < NY; ++j) {
-      const int c = tid + 256 * j, r = c / (D / 8), cc = c % (D / 8);
+      const int c = tid + 256 * j, r = c / YC, cc = c % YC;
       const int n = n0 + r;
       yr[j] = zero8<T>();
-      if (n < ny_total) yr[j] = load16<vec8>(dy + ((int64_t)n * nheads + h) * D + cc * 8);
+      if (n < ny_total) yr[j] = load16<vec8>(dy + ((int64_t)n * nheads + h) * D + dout0 + cc * 8);
     }
   };
+  find_tokens(0);
   load_step(0);
   for (int n0 = 0; n0 < ny_total; n0 += LC_KC) {
     __syncthreads();
@@ -361,7 +385,7 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
 #pragma unroll
     for (int j = 0; j < NY; ++j) {
       const int c = tid + 256 * j;
-      store16(&Ys[(c / (D / 8)) * YS + (c % (D / 8)) * 8], yr[j]);
+      store16(&Ys[(c / YC) * YS + (c % YC) * 8], yr[j]);
     }
     __syncthreads();
     if (n0 + LC_KC < ny_total) load_step(n0 + LC_KC);
@@ -381,7 +405,7 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int dd = dz + wv * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-      const int dout = t * 32 + col;
+      const int dout = dout0 + t * 32 + col;
       float v = acc[t][i];
       if (pe) v += (float)pe[((int64_t)h * ks + k) * D + dd] * dbias[h * D + dout];
       dw[(((int64_t)h * ks + k) * D + dd) * D + dout] = (T)v;
@@ -582,10 +606,23 @@ static int lc_bwd_t(const void* x, int64_t x_sn, int64_t x_sh, const void* w, co
   }
   {
     ProfScope ps_("linear_compress_dw", stream);
-    dim3 grid(ks, h, d / 128 > 0 ? d / 128 : 1);
+    dim3 grid(ks, h, d / 128);
     const T* pe_ = (const T*)pe;
-    if (d == 128) lc_dw_kernel<T, 128><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)dy, pe_, dbias, (T*)dw, cu_x, cu_y, batch, h, ks, stride);
-    else lc_dw_kernel<T, 256><<<grid, 256, 0, stream>>>((const T*)x, x_sn, x_sh, (const T*)dy, pe_, dbias, (T*)dw, cu_x, cu_y, batch, h, ks, stride);
+#define FSA_LC_DW(DD)                                                                                           \
+  {                                                                                                             \
+    constexpr int lds = LcDwLds<DD>::BYTES;                                                                     \
+    hipError_t e = hipFuncSetAttribute((const void*)lc_dw_kernel<T, DD>,                                        \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, lds);                        \
+    if (e != hipSuccess) {                                                                                      \
+      set_error("hipFuncSetAttribute(%d B LDS): %s", lds, hipGetErrorString(e));                                \
+      return (int)e;                                                                                            \
+    }                                                                                                           \
+    lc_dw_kernel<T, DD><<<grid, 256, lds, stream>>>((const T*)x, x_sn, x_sh, (const T*)dy, pe_, dbias, (T*)dw,   \
+                                                     cu_x, cu_y, batch, h, ks, stride);                         \
+  }
+    if (d == 128) FSA_LC_DW(128)
+    else FSA_LC_DW(256)
+#undef FSA_LC_DW
   }
   return 0;
 }
