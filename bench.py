@@ -173,8 +173,8 @@ def side_workload(args):
             "winattn_fwd": (4.0 * d * vis_w * hq, 2 * qbytes + kvbytes),
             "winattn_bwd_dq": (6.0 * d * vis_w * hq, 3 * qbytes + kvbytes),
             "winattn_bwd_dkdv": (8.0 * d * vis_w * hq, 2 * qbytes + 2 * kvbytes),
-            "cmp_score": (2.0 * d * vis_c * hkv, 4.0 * hkv * n * nc),                # fp32 probabilities written
-            "cmp_topk": (0.0, 4.0 * hkv * n * nc + 4.0 * hkv * n * t),               # ... read back, ids written
+            "cmp_score": (2.0 * d * vis_c * hkv, n * hkv * d * e + 4.0 * hkv * n * (nc // 4 + 1)),  # q in, fp32 block scores out
+            "cmp_topk": (0.0, 4.0 * hkv * n * (nc // 4 + 1) + 4.0 * hkv * n * t),    # ... read back, ids written
             "rope": (0.0, 2.0 * (2 * qbytes + 2 * n * hkv * d * e + 2 * nseq * nc * hkv * d * e)),  # fwd + bwd, in + out
             "gate_merge_fwd": (0.0, 4.0 * qbytes),
             "gate_merge_bwd": (0.0, 7.0 * qbytes),

@@ -41,6 +41,7 @@ struct CmpParams {
   // score / top-k
   float* score;        // [Hkv, N, score_ld]
   int64_t score_ld;
+  int rebin;           // cmp_score writes block scores (taps 1 2 2 2 1 over groups of 4 keys) instead of probabilities
 };
 
 constexpr int CMP_MODE_COMPRESSED = 0;
@@ -428,7 +429,12 @@ __global__ void win_kv_blocks_kernel(const int32_t* __restrict__ cu_q, int batch
 
 // ------------------------------------------------------------------ score ----
 // score[h, token, j] = 2^(c q[token, h*g] . ck[j, h] - lse[h*g, token]) for visible j
-template <typename T, int D>
+// REBIN (compression window of 2 strides, selection block of 4): the block scores - taps 4 b - 1 .. 4 b + 3 with
+// weights 1 2 2 2 1 - are formed in registers and written instead of the per-key probabilities, a quarter of the
+// bytes.  A lane holds groups of four consecutive keys, i.e. the last four taps of a block; the first tap is the
+// last key of the group before, which the other half of the wave holds (one exchange per group, and one value
+// carried over from the previous key tile).
+template <typename T, int D, bool REBIN>
 __global__ void __launch_bounds__(256)
 cmp_score_kernel(CmpParams p) {
   typedef typename Elem<T>::vec8 vec8;
@@ -460,7 +466,11 @@ cmp_score_kernel(CmpParams p) {
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
   float* srow = p.score + ((int64_t)h * p.n_tokens + q0 + qi) * p.score_ld;
 
-  for (int jt = 0; jt < n_keys; jt += CMP_BK) {
+  // REBIN: one more tile when the visible keys end on a tile boundary - the block that starts there still owns the
+  // last key before it
+  const int n_keys_loop = REBIN && n_keys > 0 ? n_keys + 1 : n_keys;
+  float carry = 0.f;  // REBIN, lower half of the wave: probability of the key just before this tile
+  for (int jt = 0; jt < n_keys_loop; jt += CMP_BK) {
     if (jt) __syncthreads();
     stage_kv_tile<T, D>(kbase, p.k_sn, (const T*)nullptr, 0, k0 + jt, nc - jt, Ks, (T*)nullptr, tid);
     __syncthreads();
@@ -475,8 +485,37 @@ cmp_score_kernel(CmpParams p) {
         acc[a] = Elem<T>::mfma32(kf, qreg[ks], acc[a]);
       }
     }
-    if (valid) {
-      const int limit = jmax - jt;
+    const int limit = jmax - jt;
+    if constexpr (REBIN) {
+      static_assert(NA == 2, "two 32-key halves per tile");
+      float x[NA][16], last[NA * 4], recv[NA * 4];
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+          x[a][i] = key <= limit ? fast_exp2(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
+        }
+#pragma unroll
+      for (int f = 0; f < NA * 4; ++f) {
+        last[f] = x[f >> 2][4 * (f & 3) + 3];
+        recv[f] = __shfl_xor(last[f], 32, 64);
+      }
+#pragma unroll
+      for (int f = 0; f < NA * 4; ++f) {
+        // the key before this group: the other half's group f (upper half) or f - 1 (lower half)
+        const float before = hh ? recv[f] : (f ? recv[f > 0 ? f - 1 : 0] : carry);
+        const int a = f >> 2, qd = f & 3;
+        float bsum = before;
+        bsum += 2.f * x[a][4 * qd];
+        bsum += 2.f * x[a][4 * qd + 1];
+        bsum += 2.f * x[a][4 * qd + 2];
+        bsum += x[a][4 * qd + 3];
+        const int blk = jt / 4 + a * 8 + 2 * qd + hh;
+        if (valid && blk < p.score_ld) srow[blk] = bsum;
+      }
+      carry = recv[NA * 4 - 1];
+    } else if (valid) {
 #pragma unroll
       for (int a = 0; a < NA; ++a)
 #pragma unroll
@@ -505,6 +544,7 @@ struct TopkParams {
   int hkv;
   int kernel_size, kernel_stride, block_size;
   int na, ne;           // kernel_size / kernel_stride, block_size / kernel_stride
+  int rebin;            // `score` already holds the block scores before forcing and rounding
   int nblk;             // columns of the block-score matrix: ceil(max_seqlen_q / block_size)
   int t_out;            // min(topk, nblk)
   int init_blocks, local_blocks;
@@ -542,7 +582,9 @@ cmp_topk_kernel(TopkParams p) {
   auto block_score = [&](int b) {
     float acc = 0.f;
     const int c0 = b * ne - pad;
-    if (taps_12221) {
+    if (p.rebin) {
+      acc = max(4 * b - 1, 0) < n_vis ? srow[b] : 0.f;  // blocks without a visible tap were not written
+    } else if (taps_12221) {
       const int c = 4 * b;
       f32x4 x = {0.f, 0.f, 0.f, 0.f};
       if (c + 3 < n_vis) {
@@ -719,7 +761,8 @@ template <typename T, int D>
 static int cmp_score_launch(const CmpParams& p, int batch, int hkv, int64_t max_q, hipStream_t stream) {
   ProfScope ps_("cmp_score", stream);
   dim3 grid((unsigned)((max_q + CMP_ROWS - 1) / CMP_ROWS), batch, hkv);
-  cmp_score_kernel<T, D><<<grid, 256, CMP_BK * CmpLds<D>::KS * 2, stream>>>(p);
+  if (p.rebin) cmp_score_kernel<T, D, true><<<grid, 256, CMP_BK * CmpLds<D>::KS * 2, stream>>>(p);
+  else cmp_score_kernel<T, D, false><<<grid, 256, CMP_BK * CmpLds<D>::KS * 2, stream>>>(p);
   return 0;
 }
 
@@ -895,7 +938,11 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   const int t_out = topk < nblk ? topk : nblk;
   FSA_CHECK_ARG(t_out <= 64, "fsa_cmp_topk: at most 64 blocks can be selected per query");
   FSA_CHECK_ARG(nblk * 16 <= 64 * 1024, "fsa_cmp_topk: more than 4096 selection blocks per sequence");
-  const size_t need = fsa_cmp_topk_workspace_bytes(total_q, num_kv_heads, max_seqlen_k);
+  // usual geometry (window of 2 strides, block of 4): the score kernel writes block scores, at most
+  // max_seqlen_k / 4 + 1 per query, instead of one probability per compressed key
+  const bool rebin = kernel_size == 2 * kernel_stride && block_size == 4 * kernel_stride;
+  const int64_t score_cols = rebin ? max_seqlen_k / 4 + 1 : max_seqlen_k;
+  const size_t need = fsa_cmp_topk_workspace_bytes(total_q, num_kv_heads, score_cols);
   if (!workspace || workspace_bytes < need) {
     set_error("fsa_cmp_topk: workspace too small (%zu < %zu)", workspace_bytes, need);
     return FSA_ERR_WORKSPACE;
@@ -906,7 +953,9 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   p.cu_q = cu_seqlens_q; p.cu_k = cu_seqlens_k; p.n_tokens = total_q;
   p.g = num_q_heads / num_kv_heads; p.kernel_size = kernel_size; p.kernel_stride = kernel_stride;
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * LOG2E;
-  p.score = (float*)workspace; p.score_ld = (max_seqlen_k + 3) / 4 * 4;
+  p.rebin = rebin;
+  p.score = (float*)workspace;
+  p.score_ld = (score_cols + 3) / 4 * 4;
   rc = cmp_score_dispatch(dtype, head_dim, p, batch, num_kv_heads, max_seqlen_q, stream);
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_cmp_topk score");
@@ -914,7 +963,7 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   tp.score = p.score; tp.score_ld = p.score_ld; tp.cu_q = cu_seqlens_q; tp.cu_k = cu_seqlens_k;
   tp.batch = batch; tp.n_tokens = total_q; tp.hkv = num_kv_heads;
   tp.kernel_size = kernel_size; tp.kernel_stride = kernel_stride; tp.block_size = block_size;
-  tp.na = kernel_size / kernel_stride; tp.ne = block_size / kernel_stride;
+  tp.na = kernel_size / kernel_stride; tp.ne = block_size / kernel_stride; tp.rebin = p.rebin;
   tp.nblk = nblk; tp.t_out = t_out; tp.init_blocks = init_blocks; tp.local_blocks = local_blocks;
   tp.to_bf16 = scores_to_bf16; tp.topk_idx = topk_idx; tp.block_score = block_score;
   {

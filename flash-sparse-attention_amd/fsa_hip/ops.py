@@ -235,7 +235,10 @@ def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_
     dev = q.device
     idx = torch.empty((hkv, n, t_out), dtype=torch.int32, device=dev)
     bscore = torch.empty((hkv, n, nblk), dtype=torch.float32, device=dev) if return_block_score else None
-    ws_bytes = lib.fsa_cmp_topk_workspace_bytes(n, hkv, max(1, int(max_seqlen_k)))
+    score_cols = max(1, int(max_seqlen_k))
+    if kernel_size == 2 * kernel_stride and block_size == 4 * kernel_stride:
+        score_cols = score_cols // 4 + 1  # block scores instead of per-key probabilities
+    ws_bytes = lib.fsa_cmp_topk_workspace_bytes(n, hkv, score_cols)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     lse = lse.contiguous()
     rc = lib.fsa_cmp_topk(_ptr(q), _ptr(ck), _ptr(lse), _DTYPE[q.dtype], q.stride(0), q.stride(1),

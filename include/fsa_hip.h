@@ -200,7 +200,11 @@ int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, const void* o
  *   block_score [Hkv, total_q, nblk] fp32 out, optional (NULL to skip)
  * scores_to_bf16 != 0 rounds the block scores to bf16 before the selection, as
  * the reference's per-head path does.  Equal scores are ordered by lower block id.
- * The workspace holds the fp32 probabilities.
+ * The workspace holds the fp32 probabilities, max_seqlen_k columns per query and
+ * kv head.  With kernel_size == 2 * kernel_stride and block_size == 4 * kernel_stride
+ * the block scores are formed where the probabilities are computed and only
+ * they are stored: fsa_cmp_topk_workspace_bytes(total_q, num_kv_heads,
+ * max_seqlen_k / 4 + 1) is enough then (the size for max_seqlen_k is always accepted).
  * ---------------------------------------------------------------------- */
 size_t fsa_cmp_topk_workspace_bytes(int64_t total_q, int32_t num_kv_heads, int64_t max_seqlen_k);
 

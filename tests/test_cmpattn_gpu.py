@@ -34,6 +34,8 @@ CASES = [
     ([0, 1800], 4, 2, 128, 64, 16, 64, 8, torch.bfloat16),
     ([0, 1300, 2000], 4, 2, 128, 16, 16, 32, 6, torch.float16),
     ([0, 1500], 2, 1, 64, 32, 8, 64, 8, torch.bfloat16),
+    # 64 and 128 compressed keys: the visible keys end exactly on a key tile of the score kernel
+    ([0, 1040, 3104], 4, 2, 128, 32, 16, 64, 16, torch.bfloat16),
 ]
 
 
@@ -114,6 +116,7 @@ def test_cmp_topk(dev, cu, hq, hkv, d, ks, st, bk, t, dtype):
     frac_bad = (diff > bound).float().mean().item()
     print(f"  block-score max diff {diff.max().item():.3e}, outside 2 bf16 ulp: {frac_bad:.2e}", flush=True)
     assert frac_bad < 1e-3
+    assert (diff <= 2.0 ** -6 * bs_r[~inf_r].abs() + 2e-3).all()   # no tap lost anywhere
     # 3. against the oracle end to end: rows whose k-th and (k+1)-th scores differ clearly must match
     want_e2e = orc.topk_select_ref(bs_r, t, cu, bk, to_bf16=False)
     same = (idx == want_e2e).all(-1).float().mean().item()
