@@ -55,53 +55,63 @@ template <int D> struct CmpLds {
   static constexpr int BYTES = (CMP_BK * KS + CMP_BK * VS) * 2;
 };
 
-template <typename T, int D>
-__device__ __forceinline__ void stage_kv_tile(const T* kbase, int64_t k_sn, const T* vbase, int64_t v_sn,
-                                              int row0, int n_valid, T* Ks, T* Vs, int tid) {
-  typedef typename Elem<T>::vec8 vec8;
-  constexpr int KS = CmpLds<D>::KS, VS = CmpLds<D>::VS;
-  for (int c = tid; c < CMP_BK * (D / 8); c += 256) {
-    const int row = c / (D / 8), col = c % (D / 8);
-    vec8 x = zero8<T>(), y = zero8<T>();
-    if (row < n_valid) {
-      x = load16<vec8>(kbase + (int64_t)(row0 + row) * k_sn + col * 8);
-      if (vbase) y = load16<vec8>(vbase + (int64_t)(row0 + row) * v_sn + col * 8);
-    }
-    store16(&Ks[row * KS + col * 8], x);
-    if (vbase) store16(&Vs[row * VS + col * 8], y);
-  }
-}
-
-// The same tile in two steps, so that the rows of the next tile travel while the current one is used:
-// kv_tile_load issues the global loads into registers, kv_tile_store parks them in LDS.
+// A K / V tile of CMP_BK rows travels as 16-byte chunks, chunk c = tid + 256 j of thread tid: row c / (D / 8),
+// which is tid / (D / 8) + j * ROWS_PER_STEP.  The loads are buffer loads: step j has a scalar descriptor of its
+// own (first row of the step, as many bytes as the step has rows left in the sequence) and every step uses the
+// same 32-bit lane offset (kv_tile_offset), which never changes - no per-load vector arithmetic at all, and the
+// rows past the end of the sequence (last tile only) come back as zeros from the descriptor's range check.
 template <typename T, int D> struct KvTileRegs {
-  static constexpr int N = CMP_BK * (D / 8) / 256;  // 16-byte chunks per thread and tensor
+  static constexpr int CPR = D / 8;                  // 16-byte chunks per row
+  static constexpr int ROWS_PER_STEP = 256 / CPR;
+  static constexpr int N = CMP_BK / ROWS_PER_STEP;   // chunks per thread and tensor
   typename Elem<T>::vec8 k[N], v[N];
 };
 template <typename T, int D>
-__device__ __forceinline__ void kv_tile_load(KvTileRegs<T, D>& r, const T* kbase, int64_t k_sn, const T* vbase,
-                                             int64_t v_sn, int row0, int n_valid, int tid) {
-  typedef typename Elem<T>::vec8 vec8;
+__device__ __forceinline__ uint32_t kv_tile_offset(int64_t sn, int tid) {
+  constexpr int CPR = KvTileRegs<T, D>::CPR;
+  return (uint32_t)((tid / CPR) * sn * (int64_t)sizeof(T)) + (tid % CPR) * 16;   // host: CMP_BK * sn * sizeof(T) < 2^32
+}
+template <typename T, int D, int N>
+__device__ __forceinline__ void kv_rows_load(typename Elem<T>::vec8 (&r)[N], const T* base, int64_t sn, uint32_t off,
+                                             int row0, int n_valid) {
+  constexpr int RPS = KvTileRegs<T, D>::ROWS_PER_STEP;
+  const int64_t row_bytes = sn * (int64_t)sizeof(T);
+  const char* tile = reinterpret_cast<const char*>(base) + row0 * row_bytes;
 #pragma unroll
-  for (int j = 0; j < KvTileRegs<T, D>::N; ++j) {
-    const int c = tid + 256 * j, row = c / (D / 8), col = c % (D / 8);
-    r.k[j] = zero8<T>();
-    r.v[j] = zero8<T>();
-    if (row < n_valid) {
-      r.k[j] = load16<vec8>(kbase + (int64_t)(row0 + row) * k_sn + col * 8);
-      r.v[j] = load16<vec8>(vbase + (int64_t)(row0 + row) * v_sn + col * 8);
-    }
+  for (int j = 0; j < N; ++j) {
+    const int rows = min(n_valid - j * RPS, RPS);  // rows of this step inside the sequence
+    const uint32_t bytes = rows > 0 ? (uint32_t)((rows - 1) * row_bytes) + D * (uint32_t)sizeof(T) : 0u;
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(tile + j * RPS * row_bytes), 0, (int)bytes, 0x00020000);
+    r[j] = __builtin_bit_cast(typename Elem<T>::vec8, __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0));
   }
 }
-template <typename T, int D>
+// kv_tile_load issues the global loads of a tile into registers, kv_tile_store parks them in LDS: in two steps,
+// so that the rows of the next tile can travel while the current one is used.
+template <typename T, int D, bool HAS_V = true>
+__device__ __forceinline__ void kv_tile_load(KvTileRegs<T, D>& r, const T* kbase, int64_t k_sn, uint32_t k_off,
+                                             const T* vbase, int64_t v_sn, uint32_t v_off, int row0, int n_valid,
+                                             int tid) {
+  kv_rows_load<T, D>(r.k, kbase, k_sn, k_off, row0, n_valid);
+  if (HAS_V) kv_rows_load<T, D>(r.v, vbase, v_sn, v_off, row0, n_valid);
+}
+template <typename T, int D, bool HAS_V = true>
 __device__ __forceinline__ void kv_tile_store(const KvTileRegs<T, D>& r, T* Ks, T* Vs, int tid) {
   constexpr int KS = CmpLds<D>::KS, VS = CmpLds<D>::VS;
+  constexpr int CPR = KvTileRegs<T, D>::CPR, RPS = KvTileRegs<T, D>::ROWS_PER_STEP;
 #pragma unroll
   for (int j = 0; j < KvTileRegs<T, D>::N; ++j) {
-    const int c = tid + 256 * j, row = c / (D / 8), col = c % (D / 8);
+    const int row = tid / CPR + j * RPS, col = tid % CPR;
     store16(&Ks[row * KS + col * 8], r.k[j]);
-    store16(&Vs[row * VS + col * 8], r.v[j]);
+    if (HAS_V) store16(&Vs[row * VS + col * 8], r.v[j]);
   }
+}
+template <typename T, int D, bool HAS_V = true>
+__device__ __forceinline__ void stage_kv_tile(const T* kbase, int64_t k_sn, uint32_t k_off, const T* vbase, int64_t v_sn,
+                                              uint32_t v_off, int row0, int n_valid, T* Ks, T* Vs, int tid) {
+  KvTileRegs<T, D> r;
+  kv_tile_load<T, D, HAS_V>(r, kbase, k_sn, k_off, vbase, v_sn, v_off, row0, n_valid, tid);
+  kv_tile_store<T, D, HAS_V>(r, Ks, Vs, tid);
 }
 
 // Per-row and per-work-group visible key range [lo, hi] (inclusive) in both modes.
@@ -154,6 +164,7 @@ cmpattn_fwd_kernel(CmpParams p) {
 
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
+  const uint32_t k_off = kv_tile_offset<T, D>(p.k_sn, tid), v_off = kv_tile_offset<T, D>(p.v_sn, tid);
   const T* vtr = Vs + (4 * hh + ((lane & 15) >> 2)) * VS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   float m = -INFINITY, l = 0.f;  // m in raw (unscaled) score units
@@ -165,15 +176,15 @@ cmpattn_fwd_kernel(CmpParams p) {
 
   constexpr bool PREFETCH = D <= 128;  // the next tile waits in registers where the budget allows
   KvTileRegs<T, D> nxt;
-  if (PREFETCH && jt0 < n_keys) kv_tile_load<T, D>(nxt, kbase, p.k_sn, vbase, p.v_sn, k0 + jt0, nc - jt0, tid);
+  if (PREFETCH && jt0 < n_keys) kv_tile_load<T, D>(nxt, kbase, p.k_sn, k_off, vbase, p.v_sn, v_off, k0 + jt0, nc - jt0, tid);
   for (int jt = jt0; jt < n_keys; jt += CMP_BK) {
     if (jt != jt0) __syncthreads();
     if (PREFETCH) {
       kv_tile_store<T, D>(nxt, Ks, Vs, tid);
       if (jt + CMP_BK < n_keys)
-        kv_tile_load<T, D>(nxt, kbase, p.k_sn, vbase, p.v_sn, k0 + jt + CMP_BK, nc - jt - CMP_BK, tid);
+        kv_tile_load<T, D>(nxt, kbase, p.k_sn, k_off, vbase, p.v_sn, v_off, k0 + jt + CMP_BK, nc - jt - CMP_BK, tid);
     } else {
-      stage_kv_tile<T, D>(kbase, p.k_sn, vbase, p.v_sn, k0 + jt, nc - jt, Ks, Vs, tid);
+      stage_kv_tile<T, D>(kbase, p.k_sn, k_off, vbase, p.v_sn, v_off, k0 + jt, nc - jt, Ks, Vs, tid);
     }
     __syncthreads();
     f32x16 acc[NA];
@@ -293,6 +304,7 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
 
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
   const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)h * p.v_sh;
+  const uint32_t k_off = kv_tile_offset<T, D>(p.k_sn, tid), v_off = kv_tile_offset<T, D>(p.v_sn, tid);
   const T* ktr = Ks + (4 * hh + ((lane & 15) >> 2)) * KS + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
   f32x16 dacc[NDT];
@@ -303,7 +315,7 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
 
   for (int jt = jt0; jt < n_keys; jt += CMP_BK) {
     if (jt != jt0) __syncthreads();
-    stage_kv_tile<T, D>(kbase, p.k_sn, vbase, p.v_sn, k0 + jt, nc - jt, Ks, Vs, tid);
+    stage_kv_tile<T, D>(kbase, p.k_sn, k_off, vbase, p.v_sn, v_off, k0 + jt, nc - jt, Ks, Vs, tid);
     __syncthreads();
     f32x16 acc[NA], dp[NA];
 #pragma unroll
@@ -465,6 +477,7 @@ cmp_score_kernel(CmpParams p) {
   const int n_keys = qi_last >= p.kernel_size - 1 ? min(nc, (qi_last - p.kernel_size + 1) / p.kernel_stride + 1) : 0;
   const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)h * p.k_sh;
   float* srow = p.score + ((int64_t)h * p.n_tokens + q0 + qi) * p.score_ld;
+  const uint32_t k_off = kv_tile_offset<T, D>(p.k_sn, tid);
 
   // REBIN: one more tile when the visible keys end on a tile boundary - the block that starts there still owns the
   // last key before it
@@ -472,7 +485,7 @@ cmp_score_kernel(CmpParams p) {
   float carry = 0.f;  // REBIN, lower half of the wave: probability of the key just before this tile
   for (int jt = 0; jt < n_keys_loop; jt += CMP_BK) {
     if (jt) __syncthreads();
-    stage_kv_tile<T, D>(kbase, p.k_sn, (const T*)nullptr, 0, k0 + jt, nc - jt, Ks, (T*)nullptr, tid);
+    stage_kv_tile<T, D, false>(kbase, p.k_sn, k_off, (const T*)nullptr, 0, 0u, k0 + jt, nc - jt, Ks, (T*)nullptr, tid);
     __syncthreads();
     f32x16 acc[NA];
 #pragma unroll
@@ -766,16 +779,25 @@ static int cmp_score_launch(const CmpParams& p, int batch, int hkv, int64_t max_
   return 0;
 }
 
-#define FSA_CMP_DISPATCH(FN, ...)                                                         \
+// the lane offsets inside a K / V tile are 32-bit: CMP_BK rows have to span less than 4 GiB
+static int cmp_check_strides(const CmpParams& p) {
+  const int64_t lim = ((int64_t)1 << 32) / (CMP_BK * 2);
+  FSA_CHECK_ARG(p.k_sn >= 0 && p.k_sn < lim && p.v_sn >= 0 && p.v_sn < lim,
+                "compressed / window attention: key or value row stride too large");
+  return 0;
+}
+
+#define FSA_CMP_DISPATCH(FN, P, ...)                                                      \
   do {                                                                                    \
+    if (int rc_ = cmp_check_strides(P)) return rc_;                                       \
     if (dtype == FSA_BF16) {                                                              \
-      if (head_dim == 64) return FN<__bf16, 64>(__VA_ARGS__);                             \
-      if (head_dim == 128) return FN<__bf16, 128>(__VA_ARGS__);                           \
-      if (head_dim == 256) return FN<__bf16, 256>(__VA_ARGS__);                           \
+      if (head_dim == 64) return FN<__bf16, 64>(P, __VA_ARGS__);                          \
+      if (head_dim == 128) return FN<__bf16, 128>(P, __VA_ARGS__);                           \
+      if (head_dim == 256) return FN<__bf16, 256>(P, __VA_ARGS__);                           \
     } else {                                                                              \
-      if (head_dim == 64) return FN<_Float16, 64>(__VA_ARGS__);                           \
-      if (head_dim == 128) return FN<_Float16, 128>(__VA_ARGS__);                         \
-      if (head_dim == 256) return FN<_Float16, 256>(__VA_ARGS__);                         \
+      if (head_dim == 64) return FN<_Float16, 64>(P, __VA_ARGS__);                           \
+      if (head_dim == 128) return FN<_Float16, 128>(P, __VA_ARGS__);                         \
+      if (head_dim == 256) return FN<_Float16, 256>(P, __VA_ARGS__);                         \
     }                                                                                     \
     set_error("compressed attention: head_dim=%d not supported (64, 128, 256)", head_dim); \
     return FSA_ERR_UNSUPPORTED;                                                           \
