@@ -219,8 +219,20 @@ cmpattn_fwd_kernel(CmpParams p) {
         }
     }
     mx = fmaxf(mx, xor32(mx));
-    const float mref = (mx == -INFINITY) ? 0.f : mx * p.scale_log2;
-    const float alpha = exp2f(m * p.scale_log2 - mref);  // m = -inf -> 0
+    // The reference maximum m moves only when some row of the wave outgrows it by more than 2^8: until then
+    // the probabilities are taken relative to the older, smaller maximum (at most 256, exact in the final
+    // quotient) and the accumulators need no rescaling.  (-inf) - (-inf) is NaN and compares false.
+    if (__any((mx - m) * p.scale_log2 > 8.f)) {
+      // m = -inf -> 0; a row that keeps its maximum -> 1; a row that has seen no key yet has nothing to rescale
+      const float alpha = mx == -INFINITY ? 1.f : exp2f((m - mx) * p.scale_log2);
+      l *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
+      m = mx;
+    }
+    const float mref = (m == -INFINITY) ? 0.f : m * p.scale_log2;
     float lsum = 0.f;
     vec8 pk[NJ];
 #pragma unroll
@@ -232,12 +244,9 @@ cmpattn_fwd_kernel(CmpParams p) {
         pk[a * 2 + (i >> 3)][i & 7] = (T)pv;
       }
     lsum += xor32(lsum);
-    l = l * alpha + lsum;
-    m = mx;
+    l += lsum;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[dt][i] *= alpha;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         vec8 vf = lds_read_tr8<T>(vtr + 16 * j * VS + dt * 32, 8 * VS);
@@ -295,8 +304,10 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
     doreg[ks] = load16<vec8>(dorow + ks * 8);
   }
   const int64_t stat = (int64_t)hq_i * p.n_tokens + q0 + qi;
-  const float lse_r = p.lse[stat];
-  const float delta_r = p.delta[stat];
+  // a row without any visible key has lse = -inf: +inf instead turns every probability of it into 0, not NaN
+  const float lse_in = p.lse[stat];
+  const float lse_r = lse_in == -INFINITY ? INFINITY : lse_in;
+  const float delta_s = p.delta[stat] * p.scale;
   const int jmax = KeyRange<MODE>::hi(p, qi, nc), jmin = KeyRange<MODE>::lo(p, qi);
   const int qi_first = row_lo / p.g, qi_last = (min(rows_total, row_lo + CMP_ROWS) - 1) / p.g;
   const int n_keys = KeyRange<MODE>::hi(p, qi_last, nc) + 1;                 // end of the work-group's key range
@@ -335,13 +346,23 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
     }
     const int limit = jmax - jt, limit_lo = jmin - jt;
     vec8 dsk[NJ];
+    // tiles that every row of the wave sees completely need no mask
+    if (!__all(limit >= CMP_BK - 1 && limit_lo <= 0)) {
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+          if (!(key <= limit && key >= limit_lo)) acc[a][i] = -INFINITY;
+        }
+    }
+    // dS = P (dP - delta) scale
 #pragma unroll
     for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-        const float pv = (key <= limit && key >= limit_lo) ? fast_exp2(acc[a][i] * p.scale_log2 - lse_r) : 0.f;
-        dsk[a * 2 + (i >> 3)][i & 7] = (T)(pv * (dp[a][i] - delta_r) * p.scale);
+        const float pv = fast_exp2(acc[a][i] * p.scale_log2 - lse_r);
+        dsk[a * 2 + (i >> 3)][i & 7] = (T)(pv * (dp[a][i] * p.scale - delta_s));
       }
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
