@@ -201,23 +201,19 @@ cmpattn_fwd_kernel(CmpParams p) {
     const int limit = jmax - jt, limit_lo = jmin - jt;
     float mx = m;
     // tiles that every row of the wave sees completely need no mask
-    const bool full = __all(limit >= CMP_BK - 1 && limit_lo <= 0);
-    if (full) {
-#pragma unroll
-      for (int a = 0; a < NA; ++a)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, acc[a][i]);
-    } else {
+    if (!__all(limit >= CMP_BK - 1 && limit_lo <= 0)) {
 #pragma unroll
       for (int a = 0; a < NA; ++a)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-          const float sv = (key <= limit && key >= limit_lo) ? acc[a][i] : -INFINITY;
-          acc[a][i] = sv;
-          mx = fmaxf(mx, sv);
+          if (!(key <= limit && key >= limit_lo)) acc[a][i] = -INFINITY;
         }
     }
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, acc[a][i]);
     mx = fmaxf(mx, xor32(mx));
     // The reference maximum m moves only when some row of the wave outgrows it by more than 2^8: until then
     // the probabilities are taken relative to the older, smaller maximum (at most 256, exact in the final
