@@ -51,6 +51,17 @@ def test_invalid_arguments_are_reported_not_launched():
         _lib.check(rc, "fsa_build_index")
 
 
+def test_dense_attention_refuses_row_strides_beyond_its_tile_offsets():
+    """The dense kernels address a K / V tile with 32-bit lane offsets; a row stride that does not fit is an
+    argument error, raised before anything is launched (fake, never dereferenced pointers)."""
+    lib = _lib.load()
+    fake = 0x1000
+    args = dict(dtype=0, q_sn=512, q_sh=128, k_sn=1 << 26, k_sh=128, v_sn=128, v_sh=128)
+    rc = lib.fsa_winattn_fwd(fake, fake, fake, args["dtype"], args["q_sn"], args["q_sh"], args["k_sn"], args["k_sh"],
+                             args["v_sn"], args["v_sh"], fake, 1, 64, 64, 4, 1, 128, 16, 0.1, fake, 512, 128, fake, None)
+    assert rc == -1 and b"stride" in lib.fsa_last_error()
+
+
 def test_wrappers_refuse_cpu_tensors():
     import torch
 
