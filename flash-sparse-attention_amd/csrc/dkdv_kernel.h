@@ -49,6 +49,13 @@ struct SelBwdParams {
   int window;  // sliding-window mode only
 };
 
+// Host: the kernels form q / dO row addresses with 32-bit strides - token stride and the whole span of a kv head's
+// q heads must be non-negative and below 2^31 elements.
+inline bool kv_qdo_strides_ok(const SelBwdParams& p, int head_dim) {
+  const int64_t lim = (int64_t)1 << 31;
+  return p.q_sn >= 0 && p.q_sn < lim && p.do_sn >= 0 && p.do_sn < lim && p.q_sh >= 0 && p.do_sh >= 0 &&
+         p.g * p.q_sh + head_dim < lim && p.g * p.do_sh + head_dim < lim;
+}
 
 constexpr int KV_REDUCE_SPLIT = 32;  // work-groups that share the blocks of one span in the dK/dV reduce kernel
 constexpr int KV_REDUCE_SPAN = 64;   // blocks examined by one work-group of that kernel
@@ -226,6 +233,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)h * p.g * p.q_sh;
   const T* dobase = reinterpret_cast<const T*>(p.d_o) + (int64_t)h * p.g * p.do_sh;
   const int ld_row = tid / C::CPR, ld_col = tid % C::CPR;
+  const uint32_t q_sn32 = (uint32_t)p.q_sn, q_sh32 = (uint32_t)p.q_sh, do_sn32 = (uint32_t)p.do_sn, do_sh32 = (uint32_t)p.do_sh;
 
   vec8 qst[C::CPT], dost[C::CPT];
   float lse_st = 0.f, del_st = 0.f;
@@ -247,10 +255,12 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       qst[j] = zero8<T>();
       dost[j] = zero8<T>();
       if (r < row_hi) {
-        const int trank = div_group(r, p.g, p.g_shift), head = r - trank * p.g;
-        const int token = tok_pf[j];
-        qst[j] = load16<vec8>(qbase + (int64_t)token * p.q_sn + (int64_t)head * p.q_sh + ld_col * 8);
-        dost[j] = load16<vec8>(dobase + (int64_t)token * p.do_sn + (int64_t)head * p.do_sh + ld_col * 8);
+        // row address = token * row stride + head * head stride + column: strides and the head term fit 32 bits
+        // (checked by the host), so each address is one 32 x 32 -> 64 bit multiply-add
+        const uint32_t head = p.g_shift >= 0 ? (uint32_t)(r & (p.g - 1)) : (uint32_t)(r - div_group(r, p.g, p.g_shift) * p.g);
+        const uint32_t token = (uint32_t)tok_pf[j];
+        qst[j] = load16<vec8>(qbase + ((uint64_t)token * q_sn32 + (head * q_sh32 + ld_col * 8)));
+        dost[j] = load16<vec8>(dobase + ((uint64_t)token * do_sn32 + (head * do_sh32 + ld_col * 8)));
       }
     }
     if (tid < C::KV_R) {
@@ -262,7 +272,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       if (r < row_hi) {
         const int trank = div_group(r, p.g, p.g_shift), head = r - trank * p.g;
         const int token = tok_stat;
-        const int64_t stat = (int64_t)(h * p.g + head) * p.n_tokens + token;
+        // token ids are 32-bit, so n_tokens < 2^31: one 32 x 32 -> 64 bit multiply-add
+        const uint64_t stat = (uint64_t)(uint32_t)(h * p.g + head) * (uint32_t)p.n_tokens + (uint32_t)token;
         lse_st = p.lse[stat];
         del_st = p.delta[stat];
         lim_st = blk.limit(p, token - blk.seq_start);

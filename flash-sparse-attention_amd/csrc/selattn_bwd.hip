@@ -463,6 +463,7 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   p.cu_seqlens = cu_seqlens; p.cu_blocks = cu_blocks; p.counts = counts; p.starts = starts;
   p.sel_tokens = sel_tokens;
   p.batch = batch; p.max_blocks = max_blocks; p.cap = cap; p.n_tokens = total_tokens; p.g = g; p.g_shift = group_shift(g);
+  FSA_CHECK_ARG(kv_qdo_strides_ok(p, head_dim), "fsa_selattn_bwd: q / d_o strides too large or negative");
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * LOG2E;
   p.dq_part = wsp + ws.off_dqpart;
   p.dkdv_part = (float*)(wsp + ws.off_kvpart);

@@ -145,6 +145,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   constexpr int RPI = 64 / CPR;   // rows per load / store instruction
   constexpr int NLD = 32 / RPI;   // instructions per 32-row tile
   const int srow = lane / CPR, schunk = lane % CPR;
+  const uint32_t q_sn32 = (uint32_t)p.q_sn, q_sh32 = (uint32_t)p.q_sh;
   auto row_token = [&](int sub_) {  // token id of row (sub_ + col), kept by lane col
     const int r_ = min(sub_ + col, row_hi - 1);
     return toks[div_group(r_, p.g, p.g_shift)];
@@ -155,8 +156,9 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       const int row = srow + RPI * j;
       const int tok_ = __shfl(tok_lane, row, 64);
       const int r_ = min(sub_ + row, row_hi - 1);
-      const int head_ = r_ - div_group(r_, p.g, p.g_shift) * p.g;
-      dst[j] = load16<vec8>(qbase_row + (int64_t)tok_ * p.q_sn + (int64_t)head_ * p.q_sh + schunk * 8);
+      // strides and the head term fit 32 bits (checked by the host): one 32 x 32 -> 64 bit multiply-add per row
+      const uint32_t head_ = p.g_shift >= 0 ? (uint32_t)(r_ & (p.g - 1)) : (uint32_t)(r_ - div_group(r_, p.g, p.g_shift) * p.g);
+      dst[j] = load16<vec8>(qbase_row + ((uint64_t)(uint32_t)tok_ * q_sn32 + (head_ * q_sh32 + schunk * 8)));
     }
   };
   constexpr bool STAGED = SelLds<D, BK>::STAGE_OUT;  // false: LDS cannot hold the wave tiles, direct loads / stores
@@ -174,10 +176,10 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       if (sub + SEL_WG_ROWS < row_hi) fetch_q(qst, tok_next, sub + SEL_WG_ROWS);
     } else {
       const int rc_ = min(r, row_hi - 1);
-      const int head_ = rc_ - div_group(rc_, p.g, p.g_shift) * p.g;
+      const uint32_t head_ = (uint32_t)(rc_ - div_group(rc_, p.g, p.g_shift) * p.g);
       // k-step ks contracts dims [16 ks, 16 ks + 16): the two lanes of a row read 32 contiguous bytes and a
       // cache line is used up by four consecutive loads
-      const T* qrow = qbase_row + (int64_t)token * p.q_sn + (int64_t)head_ * p.q_sh + hh * 8;
+      const T* qrow = qbase_row + ((uint64_t)(uint32_t)token * q_sn32 + (head_ * q_sh32 + hh * 8));
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) qdir[ks] = load16<vec8>(qrow + ks * 16);
     }
@@ -506,6 +508,9 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
   p.sel_tokens = sel_tokens; p.tile_prefix = tile_prefix;
   p.batch = batch; p.max_blocks = max_blocks; p.cap = total_tokens * topk; p.g = g;
   p.g_shift = group_shift(g);
+  FSA_CHECK_ARG(q_stride_n >= 0 && q_stride_n < ((int64_t)1 << 31) && q_stride_h >= 0 &&
+                    g * q_stride_h + head_dim < ((int64_t)1 << 31),
+                "fsa_selattn_fwd: q strides too large or negative");
 
   p.scale_log2 = softmax_scale * LOG2E;
   p.o_part = wsp + ws.off_opart;
