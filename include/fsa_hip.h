@@ -10,7 +10,11 @@
  *   - return value: 0 = ok, < 0 = invalid argument (see fsa_last_error()),
  *     > 0 = a hipError_t from a launch;
  *   - dtype codes: FSA_BF16 / FSA_FP16 for q, k, v, o and gradients;
- *   - strides are in ELEMENTS; the innermost (head_dim) stride is 1;
+ *   - strides are in ELEMENTS; the innermost (head_dim) stride is 1; token
+ *     and head strides are non-negative, a token stride and the span of one kv
+ *     head's group of q heads stay below 2^31 elements, and the dense
+ *     (compressed / window) kernels need 64 rows of k or v within 4 GiB -
+ *     anything else is an invalid-argument error, nothing is launched;
  *   - block ids inside topk_idx are local to the query's sequence, -1 = padding.
  *
  * The packed varlen layout is the reference's: q[N,Hq,D], k/v[N,Hkv,D],
