@@ -242,8 +242,9 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   auto fetch_tokens = [&](int base) {
 #pragma unroll
     for (int j = 0; j < C::CPT; ++j) {
-      const int r = base + ld_row + C::ROW_STEP * j;
-      tok_pf[j] = r < row_hi ? row_token(r) : 0;
+      // rows past the end of the share repeat its last row (see fetch)
+      const int r = max(min(base + ld_row + C::ROW_STEP * j, row_hi - 1), 0);
+      tok_pf[j] = row_token(r);
     }
     if (tid < C::KV_R) tok_stat = base + tid < row_hi ? row_token(base + tid) : 0;
   };
@@ -251,17 +252,14 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   auto fetch = [&](int base) {
 #pragma unroll
     for (int j = 0; j < C::CPT; ++j) {
-      const int r = base + ld_row + C::ROW_STEP * j;
-      qst[j] = zero8<T>();
-      dost[j] = zero8<T>();
-      if (r < row_hi) {
-        // row address = token * row stride + head * head stride + column: strides and the head term fit 32 bits
-        // (checked by the host), so each address is one 32 x 32 -> 64 bit multiply-add
-        const uint32_t head = p.g_shift >= 0 ? (uint32_t)(r & (p.g - 1)) : (uint32_t)(r - div_group(r, p.g, p.g_shift) * p.g);
-        const uint32_t token = (uint32_t)tok_pf[j];
-        qst[j] = load16<vec8>(qbase + ((uint64_t)token * q_sn32 + (head * q_sh32 + ld_col * 8)));
-        dost[j] = load16<vec8>(dobase + ((uint64_t)token * do_sn32 + (head * do_sh32 + ld_col * 8)));
-      }
+      // row address = token * row stride + head * head stride + column: strides and the head term fit 32 bits
+      // (checked by the host), so each address is one 32 x 32 -> 64 bit multiply-add.  Rows past the end of the
+      // share repeat its last row - values of this block's own rows, which lse = +inf turns into P = dS = 0.
+      const int r = max(min(base + ld_row + C::ROW_STEP * j, row_hi - 1), 0);
+      const uint32_t head = p.g_shift >= 0 ? (uint32_t)(r & (p.g - 1)) : (uint32_t)(r - div_group(r, p.g, p.g_shift) * p.g);
+      const uint32_t token = (uint32_t)tok_pf[j];
+      qst[j] = load16<vec8>(qbase + ((uint64_t)token * q_sn32 + (head * q_sh32 + ld_col * 8)));
+      dost[j] = load16<vec8>(dobase + ((uint64_t)token * do_sn32 + (head * do_sh32 + ld_col * 8)));
     }
     if (tid < C::KV_R) {
       const int r = base + tid;
