@@ -343,28 +343,23 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
   constexpr int NX = LC_KC * 16 / 256, NY = LC_KC * YC / 256;
   static_assert(LC_KC * YC % 256 == 0, "dY slice must divide over the threads");
   vec8 xr[NX], yr[NY];
-  // token of compressed row n at window offset k (-1 past the end); found one step before the rows are requested,
-  // so that the search through cu_y is not part of the latency of a step
-  int64_t tok_of[NX];
-  auto find_tokens = [&](int n0) {
-#pragma unroll
-    for (int j = 0; j < NX; ++j) {
-      const int n = n0 + (tid + 256 * j) / 16;
-      tok_of[j] = -1;
+  // Token of compressed row n at window offset k (-1 past the end): looked up by one thread per row of a step (a
+  // search through cu_y, a chain of dependent loads) two steps ahead and handed to the 16 threads that load the
+  // row through a small double-buffered LDS table, so the search is neither repeated per chunk nor part of the
+  // latency of a step.
+  __shared__ int tok_l[2][LC_KC];
+  auto find_tokens = [&](int n0, int buf) {
+    if (tid < LC_KC) {
+      const int n = n0 + tid;
+      int tok = -1;
       if (n < ny_total) {
         const int s = upper_seg(cu_y, batch, n);
-        tok_of[j] = cu_x[s] + (int64_t)(n - cu_y[s]) * stride + k;
+        tok = cu_x[s] + (n - cu_y[s]) * stride + k;
       }
+      tok_l[buf][tid] = tok;
     }
   };
-  auto load_step = [&](int n0) {
-#pragma unroll
-    for (int j = 0; j < NX; ++j) {  // X rows: 128 dims = 16 chunks
-      const int cc = (tid + 256 * j) % 16;
-      xr[j] = zero8<T>();
-      if (tok_of[j] >= 0) xr[j] = load16<vec8>(x + tok_of[j] * x_sn + (int64_t)h * x_sh + dz + cc * 8);
-    }
-    find_tokens(n0 + LC_KC);
+  auto load_step = [&](int n0, int buf) {
 #pragma unroll
     for (int j = 0; j < NY; ++j) {
       const int c = tid + 256 * j, r = c / YC, cc = c % YC;
@@ -372,10 +367,22 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
       yr[j] = zero8<T>();
       if (n < ny_total) yr[j] = load16<vec8>(dy + ((int64_t)n * nheads + h) * D + dout0 + cc * 8);
     }
+#pragma unroll
+    for (int j = 0; j < NX; ++j) {  // X rows: 128 dims = 16 chunks
+      const int c = tid + 256 * j, cc = c % 16;
+      const int tok = tok_l[buf][c / 16];
+      xr[j] = zero8<T>();
+      if (tok >= 0) xr[j] = load16<vec8>(x + (int64_t)tok * x_sn + (int64_t)h * x_sh + dz + cc * 8);
+    }
   };
-  find_tokens(0);
-  load_step(0);
-  for (int n0 = 0; n0 < ny_total; n0 += LC_KC) {
+  find_tokens(0, 0);
+  find_tokens(LC_KC, 1);
+  __syncthreads();
+  load_step(0, 0);
+  // step i uses table i & 1; the table of step i + 2 is written after the barriers of step i, i.e. after every
+  // thread has read the same buffer for step i's rows (in the previous iteration)
+  int buf = 0;
+  for (int n0 = 0; n0 < ny_total; n0 += LC_KC, buf ^= 1) {
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < NX; ++j) {
@@ -388,7 +395,10 @@ lc_dw_kernel(const T* __restrict__ x, int64_t x_sn, int64_t x_sh, const T* __res
       store16(&Ys[(c / YC) * YS + (c % YC) * 8], yr[j]);
     }
     __syncthreads();
-    if (n0 + LC_KC < ny_total) load_step(n0 + LC_KC);
+    if (n0 + LC_KC < ny_total) {
+      load_step(n0 + LC_KC, buf ^ 1);
+      find_tokens(n0 + 2 * LC_KC, buf);
+    }
 #pragma unroll
     for (int kk = 0; kk < LC_KC / 16; ++kk) {
       vec8 xf = lds_tr8_rows<T>(&Xs[(16 * kk + 8 * hh + tr_row) * XS + wv * 32 + tr_col], XS);  // A[m = d][k = n]
