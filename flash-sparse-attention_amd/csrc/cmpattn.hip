@@ -913,6 +913,8 @@ extern "C" int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, co
   }
   char* wsp = (char*)workspace;
   const int g = num_q_heads / num_kv_heads;
+  FSA_CHECK_ARG(kv_qdo_strides_ok(q_stride_n, q_stride_h, do_stride_n, do_stride_h, g, head_dim),
+                "fsa_cmpattn_bwd: q / d_o strides too large or negative");
   float* delta = (float*)(wsp + ws.off_delta);
   int32_t* cu_tiles = (int32_t*)(wsp + ws.off_cu_tiles);
   int32_t* counts = (int32_t*)(wsp + ws.off_counts);
@@ -938,7 +940,6 @@ extern "C" int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, co
   kv.cu_seqlens = cu_seqlens_q; kv.cu_blocks = cu_tiles; kv.counts = counts; kv.starts = nullptr;
   kv.sel_tokens = nullptr; kv.tile_prefix = tile_prefix;
   kv.batch = batch; kv.max_blocks = ws.max_blocks; kv.cap = 0; kv.n_tokens = total_q; kv.g = g; kv.g_shift = group_shift(g);
-  FSA_CHECK_ARG(kv_qdo_strides_ok(kv, head_dim), "fsa_cmpattn_bwd: q / d_o strides too large or negative");
   kv.scale = softmax_scale; kv.scale_log2 = softmax_scale * LOG2E;
   kv.dq_part = nullptr; kv.dkdv_part = (float*)(wsp + ws.off_part); kv.max_tiles = ws.max_tiles;
   kv.kv_tile_rows = kv_tile_rows(g);
@@ -1081,6 +1082,8 @@ extern "C" int fsa_winattn_bwd(const void* q, const void* k, const void* v, cons
   }
   char* wsp = (char*)workspace;
   const int g = num_q_heads / num_kv_heads;
+  FSA_CHECK_ARG(kv_qdo_strides_ok(q_stride_n, q_stride_h, do_stride_n, do_stride_h, g, head_dim),
+                "fsa_winattn_bwd: q / d_o strides too large or negative");
   float* delta = (float*)(wsp + ws.off_delta);
   int32_t* cu_tiles = (int32_t*)(wsp + ws.off_cu_tiles);
   int32_t* counts = (int32_t*)(wsp + ws.off_counts);
@@ -1105,7 +1108,6 @@ extern "C" int fsa_winattn_bwd(const void* q, const void* k, const void* v, cons
   kv.v_sn = v_stride_n; kv.v_sh = v_stride_h; kv.do_sn = do_stride_n; kv.do_sh = do_stride_h;
   kv.cu_seqlens = cu_seqlens; kv.cu_blocks = cu_tiles; kv.counts = counts; kv.tile_prefix = tile_prefix;
   kv.batch = batch; kv.max_blocks = ws.max_blocks; kv.n_tokens = total_tokens; kv.g = g; kv.g_shift = group_shift(g);
-  FSA_CHECK_ARG(kv_qdo_strides_ok(kv, head_dim), "fsa_winattn_bwd: q / d_o strides too large or negative");
   kv.scale = softmax_scale; kv.scale_log2 = softmax_scale * LOG2E;
   kv.dkdv_part = (float*)(wsp + ws.off_part); kv.max_tiles = ws.max_tiles; kv.kv_tile_rows = kv_tile_rows(g);
   kv.dk = dk; kv.dv = dv; kv.dk_sn = (int64_t)num_kv_heads * head_dim; kv.dk_sh = head_dim;

@@ -51,10 +51,10 @@ struct SelBwdParams {
 
 // Host: the kernels form q / dO row addresses with 32-bit strides - token stride and the whole span of a kv head's
 // q heads must be non-negative and below 2^31 elements.
-inline bool kv_qdo_strides_ok(const SelBwdParams& p, int head_dim) {
+inline bool kv_qdo_strides_ok(int64_t q_sn, int64_t q_sh, int64_t do_sn, int64_t do_sh, int g, int head_dim) {
   const int64_t lim = (int64_t)1 << 31;
-  return p.q_sn >= 0 && p.q_sn < lim && p.do_sn >= 0 && p.do_sn < lim && p.q_sh >= 0 && p.do_sh >= 0 &&
-         p.g * p.q_sh + head_dim < lim && p.g * p.do_sh + head_dim < lim;
+  return q_sn >= 0 && q_sn < lim && do_sn >= 0 && do_sn < lim && q_sh >= 0 && do_sh >= 0 &&
+         g * q_sh + head_dim < lim && g * do_sh + head_dim < lim;
 }
 
 constexpr int KV_REDUCE_SPLIT = 32;  // work-groups that share the blocks of one span in the dK/dV reduce kernel

@@ -428,6 +428,8 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
                  o_stride_n | o_stride_h | do_stride_n | do_stride_h) % 8 == 0,
                 "fsa_selattn_bwd: strides must be multiples of 8 elements (16-byte rows)");
   const int g = num_q_heads / num_kv_heads;
+  FSA_CHECK_ARG(kv_qdo_strides_ok(q_stride_n, q_stride_h, do_stride_n, do_stride_h, g, head_dim),
+                "fsa_selattn_bwd: q / d_o strides too large or negative");
   BwdWs ws = bwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, block_size, max_blocks);
   if (!workspace || workspace_bytes < ws.total) {
     set_error("fsa_selattn_bwd: workspace too small (%zu < %zu)", workspace_bytes, ws.total);
@@ -463,7 +465,6 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   p.cu_seqlens = cu_seqlens; p.cu_blocks = cu_blocks; p.counts = counts; p.starts = starts;
   p.sel_tokens = sel_tokens;
   p.batch = batch; p.max_blocks = max_blocks; p.cap = cap; p.n_tokens = total_tokens; p.g = g; p.g_shift = group_shift(g);
-  FSA_CHECK_ARG(kv_qdo_strides_ok(p, head_dim), "fsa_selattn_bwd: q / d_o strides too large or negative");
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * LOG2E;
   p.dq_part = wsp + ws.off_dqpart;
   p.dkdv_part = (float*)(wsp + ws.off_kvpart);

@@ -488,6 +488,10 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
                  o_stride_n | o_stride_h) % 8 == 0,
                 "fsa_selattn_fwd: strides must be multiples of 8 elements (16-byte rows)");
   const int g = num_q_heads / num_kv_heads;
+  // the kernels form q row addresses with 32-bit strides
+  FSA_CHECK_ARG(q_stride_n >= 0 && q_stride_n < ((int64_t)1 << 31) && q_stride_h >= 0 &&
+                    g * q_stride_h + head_dim < ((int64_t)1 << 31),
+                "fsa_selattn_fwd: q strides too large or negative");
   FwdWs ws = fwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, max_blocks);
   if (!workspace || workspace_bytes < ws.total) {
     set_error("fsa_selattn_fwd: workspace too small (%zu < %zu)", workspace_bytes, ws.total);
@@ -508,9 +512,6 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
   p.sel_tokens = sel_tokens; p.tile_prefix = tile_prefix;
   p.batch = batch; p.max_blocks = max_blocks; p.cap = total_tokens * topk; p.g = g;
   p.g_shift = group_shift(g);
-  FSA_CHECK_ARG(q_stride_n >= 0 && q_stride_n < ((int64_t)1 << 31) && q_stride_h >= 0 &&
-                    g * q_stride_h + head_dim < ((int64_t)1 << 31),
-                "fsa_selattn_fwd: q strides too large or negative");
 
   p.scale_log2 = softmax_scale * LOG2E;
   p.o_part = wsp + ws.off_opart;

@@ -62,6 +62,23 @@ def test_dense_attention_refuses_row_strides_beyond_its_tile_offsets():
     assert rc == -1 and b"stride" in lib.fsa_last_error()
 
 
+def test_selected_attention_refuses_q_strides_beyond_32_bits():
+    """The gathers form q / dO row addresses with 32-bit strides: a token stride of 2^31 elements is an argument
+    error of the forward and the backward entry points, raised before the workspace is looked at or anything is
+    launched (fake, never dereferenced pointers)."""
+    lib = _lib.load()
+    f = 0x1000
+    big = 1 << 31
+    rc = lib.fsa_selattn_fwd(f, f, f, 0, big, 128, 512, 128, 512, 128, f, 1, 1024, 4, 1, 128, 16, 64, 16, 0.1,
+                             f, f, f, f, f, f, 512, 128, f, f, 1 << 40, None)
+    assert rc == -1 and b"too large" in lib.fsa_last_error(), lib.fsa_last_error()
+    # q, k, v, o, d_o, lse, dtype, strides of q / k / v / o (fine) and of d_o (too large), cu_seqlens, batch,
+    # total_tokens, Hq, Hkv, D, topk, block_size, max_blocks, scale, index arrays, dq, dk, dv, workspace
+    rc = lib.fsa_selattn_bwd(f, f, f, f, f, f, 0, 512, 128, 512, 128, 512, 128, 512, 128, big, 128,
+                             f, 1, 1024, 4, 1, 128, 16, 64, 16, 0.1, f, f, f, f, f, f, f, f, f, 1 << 40, None)
+    assert rc == -1 and b"too large" in lib.fsa_last_error(), lib.fsa_last_error()
+
+
 def test_wrappers_refuse_cpu_tensors():
     import torch
 
