@@ -797,12 +797,13 @@ static int cmp_score_launch(const CmpParams& p, int batch, int hkv, int64_t max_
 }
 
 // the lane offsets inside a K / V tile are 32-bit: CMP_BK rows have to span less than 4 GiB
-static int cmp_check_strides(const CmpParams& p) {
+static int cmp_check_strides(int64_t k_sn, int64_t v_sn) {
   const int64_t lim = ((int64_t)1 << 32) / (CMP_BK * 2);
-  FSA_CHECK_ARG(p.k_sn >= 0 && p.k_sn < lim && p.v_sn >= 0 && p.v_sn < lim,
+  FSA_CHECK_ARG(k_sn >= 0 && k_sn < lim && v_sn >= 0 && v_sn < lim,
                 "compressed / window attention: key or value row stride too large");
   return 0;
 }
+static int cmp_check_strides(const CmpParams& p) { return cmp_check_strides(p.k_sn, p.v_sn); }
 
 #define FSA_CMP_DISPATCH(FN, P, ...)                                                      \
   do {                                                                                    \
@@ -915,6 +916,7 @@ extern "C" int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, co
   const int g = num_q_heads / num_kv_heads;
   FSA_CHECK_ARG(kv_qdo_strides_ok(q_stride_n, q_stride_h, do_stride_n, do_stride_h, g, head_dim),
                 "fsa_cmpattn_bwd: q / d_o strides too large or negative");
+  if (int rc_ = cmp_check_strides(k_stride_n, v_stride_n)) return rc_;
   float* delta = (float*)(wsp + ws.off_delta);
   int32_t* cu_tiles = (int32_t*)(wsp + ws.off_cu_tiles);
   int32_t* counts = (int32_t*)(wsp + ws.off_counts);
@@ -1084,6 +1086,7 @@ extern "C" int fsa_winattn_bwd(const void* q, const void* k, const void* v, cons
   const int g = num_q_heads / num_kv_heads;
   FSA_CHECK_ARG(kv_qdo_strides_ok(q_stride_n, q_stride_h, do_stride_n, do_stride_h, g, head_dim),
                 "fsa_winattn_bwd: q / d_o strides too large or negative");
+  if (int rc_ = cmp_check_strides(k_stride_n, v_stride_n)) return rc_;
   float* delta = (float*)(wsp + ws.off_delta);
   int32_t* cu_tiles = (int32_t*)(wsp + ws.off_cu_tiles);
   int32_t* counts = (int32_t*)(wsp + ws.off_counts);

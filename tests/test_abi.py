@@ -60,6 +60,11 @@ def test_dense_attention_refuses_row_strides_beyond_its_tile_offsets():
     rc = lib.fsa_winattn_fwd(fake, fake, fake, args["dtype"], args["q_sn"], args["q_sh"], args["k_sn"], args["k_sh"],
                              args["v_sn"], args["v_sh"], fake, 1, 64, 64, 4, 1, 128, 16, 0.1, fake, 512, 128, fake, None)
     assert rc == -1 and b"stride" in lib.fsa_last_error()
+    # backward: q, k, v, o, d_o, lse, dtype, strides of q / k (too large) / v / o / d_o, cu_seqlens, batch,
+    # total_tokens, max_seqlen, Hq, Hkv, D, window, scale, dq, dk, dv, workspace
+    rc = lib.fsa_winattn_bwd(fake, fake, fake, fake, fake, fake, 0, 512, 128, 1 << 26, 128, 128, 128, 512, 128, 512, 128,
+                             fake, 1, 64, 64, 4, 1, 128, 16, 0.1, fake, fake, fake, fake, 1 << 40, None)
+    assert rc == -1 and b"row stride too large" in lib.fsa_last_error(), lib.fsa_last_error()
 
 
 def test_selected_attention_refuses_q_strides_beyond_32_bits():
