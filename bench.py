@@ -62,7 +62,7 @@ def cpu_baseline(seq_len: int, d: int, bk: int, topk: int, hkv: int):
     """The CPU oracle (a PyTorch-eager port of the reference's math) timed on the host cores:
     forward + backward of the same operator on a bounded sample of the workload."""
     import torch
-    from fsa_hip.synth import make_qkv, make_topk_idx
+    from synth_inputs import make_qkv, make_topk_idx
     from oracle import selattn as orc
 
     cores = os.cpu_count() or 1
@@ -254,7 +254,7 @@ def main():
     from fsa.ops.FSA_topk_sparse_attention import (_topk_sparse_attention_bwd_opt,
                                                    _topk_sparse_attention_fwd_opt)
     from fsa_hip import _lib, ops
-    from fsa_hip.synth import make_qkv, make_topk_idx
+    from synth_inputs import make_qkv, make_topk_idx
 
     assert torch.cuda.is_available(), "bench.py needs a ROCm device"
     dev = torch.device("cuda:0")

@@ -12,7 +12,7 @@ import torch
 from fsa.ops.FSA_topk_sparse_attention import (FSA_topk_sparse_attention, _topk_sparse_attention_bwd_opt,
                                                _topk_sparse_attention_fwd_opt)
 from fsa_hip import ops
-from fsa_hip.synth import make_qkv, make_topk_idx
+from synth_inputs import make_qkv, make_topk_idx
 from oracle import selattn as orc
 
 pytestmark = pytest.mark.gpu

@@ -17,7 +17,7 @@ import pytest
 import torch
 
 from fsa_hip import ops
-from fsa_hip.synth import make_qkv, make_topk_idx
+from synth_inputs import make_qkv, make_topk_idx
 from oracle import selattn as orc
 
 pytestmark = pytest.mark.gpu

@@ -4,7 +4,7 @@ import math
 
 import torch
 
-from fsa_hip.synth import make_topk_idx
+from synth_inputs import make_topk_idx
 from oracle import cmpattn as pre
 from oracle import decode as dec
 from oracle import selattn as sel

@@ -8,7 +8,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from fsa_hip.synth import make_qkv, make_topk_idx
+from synth_inputs import make_qkv, make_topk_idx
 from oracle import selattn as orc
 
 
@@ -203,7 +203,7 @@ def test_synthetic_index_matches_stated_counts():
 def test_rows_ref_equals_chunked_oracle():
     """The per-row sampler (explicit key lists) and the chunked oracle (block views, batched gathers) agree on every
     row and on the dK/dV of every block of a small ragged batch."""
-    from fsa_hip.synth import make_qkv, make_topk_idx
+    from synth_inputs import make_qkv, make_topk_idx
     cu = [0, 150, 150, 391]
     n, hq, hkv, d, bk, t = cu[-1], 4, 2, 32, 16, 4
     q, k, v, do = make_qkv(n, hq, hkv, d, torch.float32, seed=5)
