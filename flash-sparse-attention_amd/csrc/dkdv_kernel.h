@@ -36,7 +36,7 @@ struct SelBwdParams {
   int g_shift;  // log2 g, or -1 if g is not a power of two
   float scale;
   float scale_log2;
-  void* dq_part;     // [Hkv, cap, g, D] lane-native order
+  void* dq_part;     // [Hkv, cap, g, D]
   float* dkdv_part;  // [Hkv, max_tiles, 2, BK, D]
   int64_t max_tiles;
   int kv_tile_rows;  // rows per work-group of the dK/dV kernel
@@ -111,19 +111,37 @@ static inline int kv_tile_rows(int g, int d = 128, int bk = 64) {
   return r < KV_TILE_ROWS_MAX ? r : KV_TILE_ROWS_MAX;
 }
 
+// Element offset of element `col` (a multiple of 4) of row `row` in an unpadded LDS tile with rows of W 16-bit
+// elements.  The LDS serves a half-wave (32 lanes) per cycle from 64 four-byte banks, so the 8-byte reads of a
+// half-wave must fall into distinct 16-byte slots of the 256-byte bank line.  The two read patterns of the MFMA
+// operands are 16 rows x 16 bytes (natural: row = lane % 16) and 8 rows x 32 bytes (transposing: four lanes per
+// row); with rows that are a multiple (or a fraction) of 256 bytes both would hit the same slots in every row.
+// Hence: the 32-byte group index of a row is XOR-ed with the row number (8 consecutive rows -> 8 different
+// groups), and the two 16-byte halves of every group are swapped in rows 8..15 of each 16 (16 rows x 16 bytes ->
+// 16 different slots).  Measured on gfx950 (ds_read_b64 / ds_read_b64_tr_b16, 8 waves per CU): both patterns at
+// the full rate of 1.04 ns per wave instruction, where rows padded to 272 bytes give 1.04 / 1.86 (the
+// transposing reads two-way conflicted) and rows of 288 bytes 1.86 / 1.04.
+template <int W> __device__ __forceinline__ int swz(int row, int col) {
+  static_assert(W >= 32 && (W & (W - 1)) == 0, "row length");
+  constexpr int L = W >= 128 ? 1 : 128 / W;          // rows per 256-byte bank line
+  constexpr int XM = W / 16 - 1 < 7 ? W / 16 - 1 : 7;  // 32-byte groups per row - 1, at most 8 take part
+  const int x = (row / L) & XM, hb = (row >> 3) & 1;
+  return row * W + ((((col >> 4) ^ x) << 4) | ((((col >> 3) & 1) ^ hb) << 3) | (col & 7));
+}
+
 template <int D, int BK> struct KvCfg {
   static constexpr int NW = BK / 16;        // one wave per 16 keys
   // gathered rows per pass; 32 where 8 waves of head_dim 256 leave no registers for a 64-row pass
   static constexpr int KV_R = (D >= 256 && BK >= 128) ? 32 : 64;
   static constexpr int NT = NW * 64;
-  static constexpr int QS = D + 8;         // LDS row stride of the Q / dO tiles (16 B pad; a larger pad would push two work-groups past 160 KB of LDS)
+  static constexpr int QS = D;             // LDS rows of the Q / dO tiles are unpadded and swizzled (swz<D>)
   static constexpr int CPR = D / 8;         // 16-byte chunks per row
   static constexpr int CPT = KV_R * CPR / NT;  // chunks per thread and tensor
   static constexpr int ROW_STEP = NT / CPR;
   static constexpr int BYTES = 2 * KV_R * QS * 2 + KV_R * 16;
   // with the fused dQ: K of the block (natural layout) and the dS^T tile [BK][KV_R]
-  static constexpr int KS = D + 8;
-  static constexpr int DSS = KV_R + 8;
+  static constexpr int KS = D;            // K copy: unpadded and swizzled like the Q / dO tiles
+  static constexpr int DSS = KV_R + 8;    // the small dS^T and dQ staging tiles keep padded rows
   // fused dQ: row tiles (16 rows) are dealt to the waves; with more waves than row tiles, TG waves share a
   // row tile and split its d tiles.  Each wave stages its [16][DW] piece for row-coalesced stores.
   static constexpr int NRT = KV_R / 16;
@@ -145,17 +163,14 @@ template <int D, int BK> struct KvCfg {
 // its (query, block) pairs - dQ^T = K^T dS^T with dS^T exchanged between the
 // waves through LDS - so Q and dO are gathered once for dQ, dK and dV.
 template <typename T, int D, int BK, int MODE, bool FUSE_DQ = false>
-#ifndef KV_LB_PROBE
 __global__ void __launch_bounds__((KvCfg<D, BK>::NT), (KvCfg<D, BK>::MIN_WAVES))
-#else
-__global__ void __launch_bounds__(256)
-#endif
 attn_bwd_dkdv_kernel(SelBwdParams p) {
   typedef typename Elem<T>::vec8 vec8;
   typedef typename Elem<T>::vec4 vec4;
   typedef KvCfg<D, BK> C;
   constexpr int QS = C::QS, NS = D / 32, NDT = D / 16, NRT = C::NRT, NU = C::KV_R / 32;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // aligned to the bank line and to the largest swizzled row: group addresses are formed by XOR on byte addresses
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   T* Qs = reinterpret_cast<T*>(smem);
   T* Os = Qs + C::KV_R * QS;
   float* lse_s = reinterpret_cast<float*>(Os + C::KV_R * QS);
@@ -221,7 +236,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       const int row = c / (D / 8), cc = c % (D / 8);
       vec8 x = zero8<T>();
       if (row < blk.n_keys_valid) x = load16<vec8>(kb + (int64_t)(blk.key_row0 + row) * p.k_sn + cc * 8);
-      store16(&Kl[row * C::KS + cc * 8], x);
+      store16(&Kl[swz<D>(row, cc * 8)], x);
     }
   }
   const int32_t* toks = MODE == KV_MODE_SELECTED ? p.sel_tokens + (int64_t)h * p.cap + start : nullptr;
@@ -279,12 +294,14 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       }
     }
   };
+  const int st_off = swz<D>(ld_row, ld_col * 8);
   auto stash = [&]() {
 #pragma unroll
     for (int j = 0; j < C::CPT; ++j) {
-      const int row = ld_row + C::ROW_STEP * j;
-      store16(&Qs[row * QS + ld_col * 8], qst[j]);
-      store16(&Os[row * QS + ld_col * 8], dost[j]);
+      // the swizzle of a row repeats every 16 rows
+      const int off = C::ROW_STEP % 16 == 0 ? st_off + C::ROW_STEP * j * QS : swz<D>(ld_row + C::ROW_STEP * j, ld_col * 8);
+      store16(&Qs[off], qst[j]);
+      store16(&Os[off], dost[j]);
     }
     if (tid < C::KV_R) {
       lse_s[tid] = lse_st;
@@ -304,8 +321,14 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     }
 
   // lane addresses: A operand rows (natural) and transposing reads
-  const int a_off = l16 * QS + (SPLIT ? 4 : 8) * kg;              // + rt*16*QS + 32*s (SPLIT: + 16 for the second half)
-  const int tr_off = (4 * kg + (l16 >> 2)) * QS + 4 * (l16 & 3);  // + 32*u*QS + 16*dtile
+  // The row part of a swizzled offset repeats every 16 rows and the 32-byte group g of a row sits at the
+  // offset of group 0 XOR 16 g elements, so a lane keeps one offset per access pattern:
+  // byte addresses inside the Q tile, 32-byte group 0: the row part of a swizzled offset repeats every 16 rows,
+  // and group g of a row sits at the address of group 0 XOR 32 g (the tiles start on multiples of the row size)
+  const uint32_t a_addr00 = lds_addr(Qs + swz<D>(l16, (SPLIT ? 4 : 8) * kg));            // + rt*16 rows
+  const uint32_t tr_addr00 = lds_addr(Qs + swz<D>(4 * kg + (l16 >> 2), 4 * (l16 & 3)));  // + 32*u rows (+ 16 rows)
+  constexpr int ROW_BYTES = QS * 2, O_BYTES = C::KV_R * ROW_BYTES;                        // Os - Qs
+  constexpr int K_BYTES = 2 * O_BYTES + C::KV_R * 16;                                     // Kl - Qs
 
 
   fetch_tokens(row_lo);
@@ -315,6 +338,10 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   __syncthreads();
   for (int base = row_lo; base < row_hi; base += C::KV_R) {
     const bool more = base + C::KV_R < row_hi;
+    // The per-group offsets (offset of group 0 XOR a constant) are formed where they are used: computed once
+    // before the loop they would occupy some twenty registers for the whole kernel.
+    uint32_t a_addr0 = a_addr00, tr_addr0 = tr_addr00;
+    asm volatile("" : "+v"(a_addr0), "+v"(tr_addr0));
     if (more) {
       fetch(base + C::KV_R);
       fetch_tokens(base + 2 * C::KV_R);
@@ -329,9 +356,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     // limit 2-3 (| lower limit 0-1 | 2-3 in window mode)]
     constexpr int NST = RAW ? (MODE == KV_MODE_WINDOW ? 8 : 6) : 1;
     u32x2 st[2][NST];
-    const uint32_t a_addr = lds_addr(Qs + a_off);
     const uint32_t s_addr = lds_addr(lse_s + 4 * kg);
-    constexpr int O_BYTES = C::KV_R * QS * 2;  // Os - Qs
     constexpr int STAT_BYTES = C::KV_R * 4;    // del_s - lse_s = lim_s - del_s = llo_s - lim_s
     // compiler-issued path: k-steps outside, row tiles inside, so that a K fragment that comes from LDS is read
     // once per pass
@@ -344,12 +369,12 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       }
 #pragma unroll
       for (int s_ = 0; s_ < NS; ++s_) {
-        const vec8 kfrag = KLDS ? load16<vec8>(&Kl[key * C::KS + 32 * s_ + 8 * kg]) : kf[KLDS ? 0 : s_];
+        const vec8 kfrag = KLDS ? load16<vec8>(&Kl[swz<D>(key, 32 * s_ + 8 * kg)]) : kf[KLDS ? 0 : s_];
 #pragma unroll
         for (int rt = 0; rt < NRT; ++rt) {
-          vec8 qa = load16<vec8>(&Qs[rt * 16 * QS + a_off + 32 * s_]);
+          vec8 qa = load16<vec8>(lds_ptr<T>((a_addr0 ^ (64u * s_)) + rt * 16 * ROW_BYTES));
           sacc_all[rt] = Elem<T>::mfma16(qa, kfrag, sacc_all[rt]);
-          vec8 da = load16<vec8>(&Os[rt * 16 * QS + a_off + 32 * s_]);
+          vec8 da = load16<vec8>(lds_ptr<T>((a_addr0 ^ (64u * s_)) + (O_BYTES + rt * 16 * ROW_BYTES)));
           dpacc_all[rt] = Elem<T>::mfma16(da, vf[s_], dpacc_all[rt]);
         }
         if (C::TIGHT_REGS && (s_ & 1) == 1) asm volatile("" ::: "memory");
@@ -367,25 +392,15 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
           if (a_ == 2) { sd[4] = lds_read8_raw<2 * STAT_BYTES + rt * 64>(s_addr); sd[5] = lds_read8_raw<2 * STAT_BYTES + rt * 64 + 8>(s_addr); }
           if (a_ == 3) { sd[NST - 2] = lds_read8_raw<3 * STAT_BYTES + rt * 64>(s_addr); sd[NST - 1] = lds_read8_raw<3 * STAT_BYTES + rt * 64 + 8>(s_addr); }
         }
-        dst[0] = lds_read8_raw<RB>(a_addr);
-        dst[NS] = lds_read8_raw<RB + 32>(a_addr);
-        dst[2 * NS] = lds_read8_raw<O_BYTES + RB>(a_addr);
-        dst[3 * NS] = lds_read8_raw<O_BYTES + RB + 32>(a_addr);
-        if constexpr (NS > 1) {
-          dst[1] = lds_read8_raw<RB + 64>(a_addr);
-          dst[NS + 1] = lds_read8_raw<RB + 96>(a_addr);
-          dst[2 * NS + 1] = lds_read8_raw<O_BYTES + RB + 64>(a_addr);
-          dst[3 * NS + 1] = lds_read8_raw<O_BYTES + RB + 96>(a_addr);
-        }
-        if constexpr (NS > 2) {
-          dst[2] = lds_read8_raw<RB + 128>(a_addr);
-          dst[NS + 2] = lds_read8_raw<RB + 160>(a_addr);
-          dst[2 * NS + 2] = lds_read8_raw<O_BYTES + RB + 128>(a_addr);
-          dst[3 * NS + 2] = lds_read8_raw<O_BYTES + RB + 160>(a_addr);
-          dst[3] = lds_read8_raw<RB + 192>(a_addr);
-          dst[NS + 3] = lds_read8_raw<RB + 224>(a_addr);
-          dst[2 * NS + 3] = lds_read8_raw<O_BYTES + RB + 192>(a_addr);
-          dst[3 * NS + 3] = lds_read8_raw<O_BYTES + RB + 224>(a_addr);
+        uint32_t a_addr = a_addr0;
+        asm volatile("" : "+v"(a_addr));  // the group addresses are formed per row tile, next to their reads
+#pragma unroll
+        for (int s_ = 0; s_ < NS; ++s_) {  // group 2 s_ holds the first, group 2 s_ + 1 the second half of k-step s_
+          const uint32_t lo = a_addr ^ (64u * s_), hi = a_addr ^ (64u * s_ + 32u);
+          dst[s_] = lds_read8_raw<RB>(lo);
+          dst[NS + s_] = lds_read8_raw<RB>(hi);
+          dst[2 * NS + s_] = lds_read8_raw<O_BYTES + RB>(lo);
+          dst[3 * NS + s_] = lds_read8_raw<O_BYTES + RB>(hi);
         }
       }
     };
@@ -458,9 +473,10 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       vec8 dsb = __builtin_shufflevector(dsk[2 * u], dsk[2 * u + 1], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
       for (int t = 0; t < NDT; ++t) {
-        vec8 doa = lds_read_tr8<T>(&Os[32 * u * QS + tr_off + 16 * t], 16 * QS);
+        const T* trp = lds_ptr<T>(tr_addr0 ^ (32u * t));
+        vec8 doa = lds_read_tr8<T>(trp + (O_BYTES / 2 + 32 * u * QS), 16 * QS);
         dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
-        vec8 qa = lds_read_tr8<T>(&Qs[32 * u * QS + tr_off + 16 * t], 16 * QS);
+        vec8 qa = lds_read_tr8<T>(trp + 32 * u * QS, 16 * QS);
         dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
         if (C::TIGHT_REGS && (t & 1) == 1) asm volatile("" ::: "memory");  // keep the operand reads from piling up
       }
@@ -470,7 +486,6 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       // dealt round-robin to the waves, both operands come from transposing LDS reads
       T* dqpart = reinterpret_cast<T*>(p.dq_part);
       const int64_t prow0 = ((int64_t)h * p.cap + start) * p.g;
-      const int ktr_off = (4 * kg + (l16 >> 2)) * C::KS + 4 * (l16 & 3);   // + 32*u*KS + 16*t
       const int str_off = (4 * kg + (l16 >> 2)) * C::DSS + 4 * (l16 & 3);  // + 32*u*DSS + 16*rt
       const int tg = wv / C::RW;                     // which share of the d tiles
       constexpr int NTW = NDT / C::TG;               // d tiles per wave
@@ -485,7 +500,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int u = 0; u < BK / 32; ++u) {
-            vec8 ka = lds_read_tr8<T>(&Kl[32 * u * C::KS + ktr_off + 16 * t], 16 * C::KS);
+            // the K copy is swizzled like the Q tile (same row pattern)
+            vec8 ka = lds_read_tr8<T>(lds_ptr<T>(tr_addr0 ^ (32u * t)) + (K_BYTES / 2 + 32 * u * C::KS), 16 * C::KS);
             acc = Elem<T>::mfma16(ka, dsb[u], acc);
           }
           vec4 x;

@@ -91,6 +91,10 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint32_t lds_addr(const void* p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
+// the LDS pointer for a byte address
+template <typename T> __device__ __forceinline__ const T* lds_ptr(uint32_t addr) {
+  return (const T*)(__attribute__((address_space(3))) const T*)(uintptr_t)addr;
+}
 template <int OFFSET_BYTES> __device__ __forceinline__ u32x2 lds_read8_raw(uint32_t addr) {
   static_assert(OFFSET_BYTES >= 0 && OFFSET_BYTES < 65536, "ds offset field");
   u32x2 r;
