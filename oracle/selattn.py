@@ -15,6 +15,9 @@ Pinning status (tests/test_oracle_selattn.py):
       selected_attention_ref and central finite differences on tiny inputs.
   selected_attention_rows_ref : pinned - equals the two functions above on
       every row / block of small inputs (independent code path).
+  key_block_grads_ref : pinned - equals selected_attention_rows_ref
+      (key_block=...) summed over every query that selected the block, on small
+      inputs, and the dK / dV slices of selected_attention_grads_ref.
   build_index_ref : pinned - brute-force Python loops, torch.bincount,
       exclusive cumsum identity.
 """
@@ -247,6 +250,49 @@ def selected_attention_rows_ref(q, k, v, topk_idx, block_size, cu_seqlens, rows,
                     out["dk_block"][off] += ds_c[:, inblk].t() @ q[row, hs].to(dtype)
                     out["dv_block"][off] += p_c[:, inblk].t() @ dor
     return out
+
+
+def key_block_grads_ref(q, k, v, do, o_in, lse_in, kv_head: int, block_row0: int, users, block_size: int,
+                        seq_end: int, softmax_scale=None, round_dtype=None, dtype=torch.float64, chunk: int = 8192):
+    """dK, dV [B_K, D] of ONE key block (kv head `kv_head`, first global row `block_row0`) from ALL the queries
+    in `users` (global rows of the queries that selected the block), vectorised so that a block selected by every
+    query of a 64K sequence is cheap.  The backward operator takes the stored forward output and LSE as inputs
+    (FSA_topk_sparse_attention.py:1715-1730), so o_in [N, Hq, D] and lse_in [Hq, N] (base 2) are required:
+    P = 2^(c q.k - LSE2) for key row <= query row (:520), delta = sum_d O dO, dS = scale * P * (dO.v - delta),
+    dK = sum dS^T q, dV = sum P^T dO over the users and the g heads of the group (:1697-1709, 1854-1855), with P
+    and dS cast to round_dtype before the second products when given (:1705-1706).  Rows of the block at or past
+    seq_end are zero."""
+    def rnd(x):
+        return x if round_dtype is None else x.to(round_dtype).to(dtype)
+
+    N, Hq, D = q.shape
+    g = Hq // k.shape[1]
+    B = block_size
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    c = softmax_scale * LOG2E
+    nk = min(B, seq_end - block_row0)
+    kk = k[block_row0 : block_row0 + nk, kv_head].to(dtype)          # [nk, D]
+    vv = v[block_row0 : block_row0 + nk, kv_head].to(dtype)
+    hs = slice(kv_head * g, (kv_head + 1) * g)
+    users = torch.as_tensor(users, dtype=torch.long)
+    dk = torch.zeros(B, D, dtype=dtype)
+    dv = torch.zeros(B, D, dtype=dtype)
+    key_rows = block_row0 + torch.arange(nk)
+    for u0 in range(0, users.numel(), chunk):
+        u = users[u0 : u0 + chunk]
+        qr, dor, orr = (x[u][:, hs].to(dtype) for x in (q, do, o_in))   # [C, g, D]
+        lse = lse_in[hs][:, u].to(dtype).t()[:, :, None]                # [C, g, 1]
+        sc = torch.einsum("cgd,kd->cgk", qr, kk) * c
+        vis = (key_rows[None, :] <= u[:, None])[:, None, :]             # [C, 1, nk]
+        p = torch.where(vis, torch.exp2(sc - lse), torch.zeros((), dtype=dtype))
+        dp = torch.einsum("cgd,kd->cgk", dor, vv)
+        delta = (orr * dor).sum(-1, keepdim=True)
+        ds = softmax_scale * p * (dp - delta)
+        ds_c, p_c = rnd(ds), rnd(p)
+        dk[:nk] += torch.einsum("cgk,cgd->kd", ds_c, qr)
+        dv[:nk] += torch.einsum("cgk,cgd->kd", p_c, dor)
+    return dk, dv
 
 
 def dense_mask(topk_idx: torch.Tensor, block_size: int, cu_seqlens) -> torch.Tensor:

@@ -3,6 +3,8 @@
 * index lists bit-exact against the CPU oracle (a sort of N*T keys, cheap at any size);
 * O / LSE / dQ of a seeded SAMPLE of queries, and dK / dV of sampled key blocks, against the per-row oracle
   (same tolerances as the small cases: 2e-2 bf16, 5e-3 fp16, LSE 1e-3, plus one output ulp for gradients);
+* dK / dV of block 0 - selected by every query, the one block whose rows are dealt to many work-groups and whose
+  fp32 partials meet in the reduce kernel - element by element against the vectorised per-block oracle;
 * size-independent identities over the WHOLE output:
     - scaling V by 2 scales O by exactly 2 and leaves LSE bit-identical (powers of two commute with rounding
       outside the subnormal range; bit-exact for bf16, one ulp for fp16);
@@ -28,6 +30,7 @@ ULP = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}
 CASES = [
     # name, S, Hq, Hkv, D, B_K, T, dtype, std
     ("C1-gqa4", 65536, 16, 4, 128, 64, 16, torch.bfloat16, 1.0),
+    ("C1-gqa2", 65536, 8, 4, 128, 64, 16, torch.bfloat16, 1.0),
     ("C1-gqa1", 65536, 4, 4, 128, 64, 16, torch.bfloat16, 1.0),
     ("C3", 131072, 4, 2, 256, 128, 8, torch.float16, 0.5),
 ]
@@ -89,8 +92,22 @@ def test_selected_attention_full_size(dev, name, n, hq, hkv, d, bk, t, dtype, st
     print(f"  sampled rows: max|dO|={eo:.3e} max|dLSE|={el:.3e} dQ excess={edq:.3e}", flush=True)
     assert eo <= TOL[dtype] and el <= 1e-3 and edq <= TOL[dtype]
 
-    # sampled key blocks (block 0 has every query: too many rows for the CPU; take moderately shared blocks)
+    # block 0: every query selects it (N * g rows, many work-groups, fp32 partials + reduce kernel)
     nblk = (n + bk - 1) // bk
+    worst = {"dk": 0.0, "dv": 0.0}
+    for kh in sorted({0, hkv - 1}):
+        users = sel_tokens[kh][: int(counts[kh, 0])]
+        assert len(users) == n
+        dk0, dv0 = orc.key_block_grads_ref(q, k, v, do, oc, lc, kh, 0, users, bk, n, round_dtype=dtype)
+        for nm, got, want in (("dk", dk, dk0), ("dv", dv, dv0)):
+            gb = got[:bk, kh].float().cpu().double()
+            err = (gb - want).abs().max().item()
+            ex = ((gb - want).abs() - ULP[dtype] * want.abs()).max().item()
+            worst[nm] = max(worst[nm], err)
+            print(f"  block 0 kv head {kh} ({n} queries): {nm} max err {err:.3e} (|ref| max {want.abs().max().item():.1f})", flush=True)
+            assert ex <= TOL[dtype], (nm, 0, ex)
+
+    # moderately shared key blocks through the per-row oracle
     for kh, blk in [(0, nblk // 8), (hkv - 1, nblk // 2), (0, nblk - 1)]:
         s0 = int(starts[kh, blk])
         users = sel_tokens[kh][s0 : s0 + int(counts[kh, blk])].tolist()
@@ -99,8 +116,12 @@ def test_selected_attention_full_size(dev, name, n, hq, hkv, d, bk, t, dtype, st
         for nm, got, want in (("dk", dk, rb["dk_block"]), ("dv", dv, rb["dv_block"])):
             gb = got[blk * bk : (blk + 1) * bk, kh].float().cpu().double()
             ex = ((gb - want).abs() - ULP[dtype] * want.abs()).max().item()
+            worst[nm] = max(worst[nm], (gb - want).abs().max().item())
             print(f"  block {blk} kv head {kh} ({len(users)} queries): {nm} max err {(gb - want).abs().max().item():.3e}", flush=True)
             assert ex <= TOL[dtype], (nm, blk, ex)
+    edq_abs = (dqg - r["dq"]).abs().max().item()
+    print(f"MAXABS {name}: O {eo:.2e} LSE {el:.2e} dQ {edq_abs:.2e} dK {worst['dk']:.2e} dV {worst['dv']:.2e} "
+          f"(sampled rows / blocks incl. block 0)", flush=True)
 
 
 def test_decode_full_size(dev):

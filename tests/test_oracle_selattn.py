@@ -217,3 +217,33 @@ def test_rows_ref_equals_chunked_oracle():
         hi = min(first + bk, 150 if first < 150 else n)
         assert torch.allclose(r["dk_block"][: hi - first], dk[first:hi, kh], atol=1e-9)
         assert torch.allclose(r["dv_block"][: hi - first], dv[first:hi, kh], atol=1e-9)
+
+
+def test_key_block_grads_ref_equals_other_oracles():
+    """The vectorised per-block dK / dV (used for blocks that every query selects) equals the chunked oracle's
+    slices and the per-row sampler, with and without the kernels' rounding points, including a block cut by the
+    sequence end and a stored (perturbed) O / LSE as inputs."""
+    from synth_inputs import make_qkv, make_topk_idx
+    cu = [0, 150, 150, 391]
+    n, hq, hkv, d, bk, t = cu[-1], 4, 2, 32, 16, 4
+    q, k, v, do = make_qkv(n, hq, hkv, d, torch.float32, seed=15)
+    idx = make_topk_idx(cu, hkv, bk, t, seed=16)
+    o, lse, _, dk, dv = orc.selected_attention_grads_ref(q, k, v, idx, bk, cu, do, dtype=torch.float64)
+    _, _, starts, sel_tokens, _ = orc.build_index_ref(idx, cu, bk)
+    cases = [(0, 0, 0, 150), (1, 150, 10, 391), (1, 150 + 15 * bk, 25, 391), (0, 9 * bk, 9, 150)]
+    for kh, first, gb, seq_end in cases:
+        users = sel_tokens[kh, int(starts[kh, gb]):int(starts[kh, gb + 1])].tolist()
+        assert users, "block without users"
+        dk_b, dv_b = orc.key_block_grads_ref(q, k, v, do, o, lse, kh, first, users, bk, seq_end, chunk=37)
+        hi = min(first + bk, seq_end)
+        assert torch.allclose(dk_b[: hi - first], dk[first:hi, kh], atol=1e-9)
+        assert torch.allclose(dv_b[: hi - first], dv[first:hi, kh], atol=1e-9)
+        assert (dk_b[hi - first:] == 0).all() and (dv_b[hi - first:] == 0).all()
+        # stored, perturbed forward results as inputs + bf16 rounding points: against the per-row sampler
+        o_in = (o + 0.01 * torch.sin(torch.arange(o.numel(), dtype=torch.float64)).view_as(o))
+        lse_in = lse + 0.003
+        r = orc.selected_attention_rows_ref(q, k, v, idx, bk, cu, users, do=do, o_in=o_in, lse_in=lse_in,
+                                            round_dtype=torch.bfloat16, key_block=(kh, first))
+        dk_b, dv_b = orc.key_block_grads_ref(q, k, v, do, o_in, lse_in, kh, first, users, bk, seq_end,
+                                             round_dtype=torch.bfloat16)
+        assert torch.allclose(dk_b, r["dk_block"], atol=1e-9) and torch.allclose(dv_b, r["dv_block"], atol=1e-9)
