@@ -25,6 +25,8 @@
 // fsa_preview/ops/selected_attention_decode.py:8-42.
 #include "fsa_common.h"
 
+#include <mutex>
+
 namespace fsa {
 
 constexpr int DEC_MODE_COMPRESSED = 0;
@@ -522,6 +524,38 @@ static size_t dec_ws_bytes(int batch, int hq, int hkv, int d) {
   return dec_ws_prefix_bytes(batch) + ((size_t)DEC_MAX_WAVES + (size_t)batch * hkv) * (hq / hkv) * (4 + d) * 4;
 }
 
+// Scratch memory of fsa_decode_selattn_static: lives in the code object, one copy per device that loads it, for
+// as long as the process runs.  In host code the array's name is only a handle for hipGetSymbolAddress.
+constexpr size_t DEC_STATIC_SCRATCH_BYTES = (size_t)FSA_DECODE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char dec_static_scratch[DEC_STATIC_SCRATCH_BYTES];
+
+// Device address of the scratch array on the current device; looked up once per device.
+static int dec_static_scratch_ptr(void** out) {
+  constexpr int MAX_DEV = 64;
+  static void* ptr[MAX_DEV] = {nullptr};
+  static std::mutex mu;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("fsa_decode_selattn_static: hipGetDevice: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (dev >= 0 && dev < MAX_DEV && ptr[dev]) {
+    *out = ptr[dev];
+    return 0;
+  }
+  void* a = nullptr;
+  e = hipGetSymbolAddress(&a, HIP_SYMBOL(dec_static_scratch));
+  if (e != hipSuccess || !a) {
+    set_error("fsa_decode_selattn_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    return e != hipSuccess ? (int)e : FSA_ERR_UNSUPPORTED;
+  }
+  if (dev >= 0 && dev < MAX_DEV) ptr[dev] = a;
+  *out = a;
+  return 0;
+}
+
 }  // namespace fsa
 
 using namespace fsa;
@@ -624,4 +658,31 @@ extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_decode_selattn");
   return 0;
+}
+
+extern "C" int fsa_decode_selattn_static(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
+                                         int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n,
+                                         int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
+                                         const int32_t* cu_k, const int32_t* topk_idx, int32_t batch,
+                                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                         int32_t topk, int32_t block_size, float softmax_scale, void* o,
+                                         float* lse, void* stream_) {
+  FSA_CHECK_ARG(batch >= 1 && num_kv_heads >= 1 && num_q_heads >= 1 && num_q_heads % num_kv_heads == 0 &&
+                    head_dim >= 1,
+                "fsa_decode_selattn_static: bad sizes");
+  const size_t need = dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim);
+  if (need > DEC_STATIC_SCRATCH_BYTES) {
+    set_error("fsa_decode_selattn_static: batch %d x %d kv heads x %d heads per group x head_dim %d needs %zu bytes "
+              "of scratch, the built-in buffer holds %zu; use fsa_decode_selattn with a caller workspace",
+              batch, num_kv_heads, num_q_heads / num_kv_heads, head_dim, need, DEC_STATIC_SCRATCH_BYTES);
+    return FSA_ERR_WORKSPACE;
+  }
+  void* scratch = nullptr;
+  int rc = dec_static_scratch_ptr(&scratch);
+  if (rc) return rc;
+  // every partial slot that the merge reads is written by the attention kernel of the same call: nothing in the
+  // buffer has to start at zero
+  return fsa_decode_selattn(q, k_cache, v_cache, dtype, q_stride_b, q_stride_h, k_stride_n, k_stride_h, v_stride_n,
+                            v_stride_h, cu_k, topk_idx, batch, num_q_heads, num_kv_heads, head_dim, topk, block_size,
+                            softmax_scale, o, lse, scratch, DEC_STATIC_SCRATCH_BYTES, stream_);
 }

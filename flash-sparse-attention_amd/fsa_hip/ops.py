@@ -326,6 +326,31 @@ def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scal
     return o, lse
 
 
+def decode_selattn_static(q, k_cache, v_cache, cu_k, topk_idx, block_size, o, lse, softmax_scale=None):
+    """Decode-step selected attention into caller-provided `o` [B,Hq,D] and `lse` [Hq,B], with the partial results
+    in the library's built-in scratch buffer: the call allocates nothing (C entry point fsa_decode_selattn_static).
+    Raises if the sizes exceed the buffer."""
+    _require_cuda(q, k_cache, v_cache, cu_k, topk_idx, o, lse)
+    assert q.dtype in _DTYPE and q.dtype == k_cache.dtype == v_cache.dtype == o.dtype
+    assert topk_idx.dtype == torch.int32 and topk_idx.is_contiguous()
+    assert q.stride(2) == 1 and k_cache.stride(2) == 1 and v_cache.stride(2) == 1
+    assert o.is_contiguous() and lse.is_contiguous() and lse.dtype == torch.float32
+    lib = _lib.load()
+    b, hq, d = q.shape
+    hkv = k_cache.shape[1]
+    assert topk_idx.shape[0] == hkv and topk_idx.shape[1] == b
+    assert o.shape == (b, hq, d) and lse.shape == (hq, b)
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(d)
+    rc = lib.fsa_decode_selattn_static(_ptr(q), _ptr(k_cache), _ptr(v_cache), _DTYPE[q.dtype], q.stride(0),
+                                       q.stride(1), k_cache.stride(0), k_cache.stride(1), v_cache.stride(0),
+                                       v_cache.stride(1), _ptr(cu_k), _ptr(topk_idx), b, hq, hkv, d,
+                                       topk_idx.shape[2], block_size, float(softmax_scale), _ptr(o), _ptr(lse),
+                                       _stream(q.device))
+    _lib.check(rc, "fsa_decode_selattn_static")
+    return o, lse
+
+
 def winattn_fwd(q, k, v, cu_seqlens, max_seqlen, window, softmax_scale=None):
     """Causal sliding-window attention (keys i-window..i): (o, lse [Hq,N] fp32 base 2)."""
     _check_qkv(q, k, v)

@@ -286,6 +286,25 @@ int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, 
                        int32_t head_dim, int32_t topk, int32_t block_size, float softmax_scale, void* o,
                        float* lse, void* workspace, size_t workspace_bytes, void* stream);
 
+/* fsa_decode_selattn for callers that cannot allocate (a step recorded into a HIP
+ * graph, a serving loop with a fixed memory plan, a harness that forbids
+ * allocation): same arguments and results as fsa_decode_selattn, but the partial
+ * results live in a buffer of FSA_DECODE_STATIC_SCRATCH_BYTES that is part of the
+ * library's code object (each device the library runs on holds its copy until the
+ * process ends), and the call allocates nothing.  No counterpart in the
+ * reference.  Sizes with fsa_decode_workspace_bytes(...) above the buffer are
+ * refused with FSA_ERR_WORKSPACE.  All calls on one device share the buffer:
+ * calls that overlap on a device (different streams or threads) race; calls on
+ * one stream do not.  The first call on a device looks the buffer up
+ * (hipGetSymbolAddress); make it outside a stream capture. */
+#define FSA_DECODE_STATIC_SCRATCH_BYTES (16u << 20)
+int fsa_decode_selattn_static(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
+                              int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
+                              int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_k,
+                              const int32_t* topk_idx, int32_t batch, int32_t num_q_heads,
+                              int32_t num_kv_heads, int32_t head_dim, int32_t topk, int32_t block_size,
+                              float softmax_scale, void* o, float* lse, void* stream);
+
 /* ------------------------------------------------------------------------
  * Sliding-window attention: the query at sequence-local position i attends the
  * keys p with i - window <= p <= i of its own sequence (window + 1 keys).
