@@ -24,19 +24,37 @@ sys.path.insert(0, os.path.join(ROOT, "flash-sparse-attention_amd"))
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense bf16/fp16
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 
-# HBM bytes per launch at the default workload from two rocprofv3 --pmc passes over this script
-# (FETCH_SIZE, WRITE_SIZE; KiB per dispatch), each scaled by the factor that makes the same counter
-# read 1 GiB for the 1 GiB device copy of --calib-copy (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).
-PMC_TRAFFIC_BYTES = {
-    ("selattn_bwd_dqdkdv", 4): 13549486080,
-    ("selattn_bwd_dqdkdv", 2): 6610281472,
-    ("selattn_bwd_dqdkdv", 1): 3254586368,
-    ("selattn_fwd_main", 4): 8274831360,
-    ("selattn_fwd_main", 2): 4033090560,
-    ("selattn_fwd_main", 1): 1987578880,
-    ("selattn_fwd_reduce", 4): 4978273280,
-    ("selattn_bwd_dq_reduce", 4): 4650569728,
-}
+# Kernels whose least work is a dense 16-bit contraction are priced against the MFMA peak (with the HBM view
+# beside it), the streaming / gathering / integer kernels against the HBM peak.
+MFMA_KERNELS = {"selattn_fwd_main", "selattn_bwd_dqdkdv", "cmpattn_fwd", "cmpattn_bwd_dq", "cmpattn_bwd_dkdv",
+                "winattn_fwd", "winattn_bwd_dq", "winattn_bwd_dkdv", "cmp_score", "linear_compress_fwd",
+                "linear_compress_dx", "linear_compress_dw"}
+
+# Measured HBM traffic per launch comes from the committed counter summary of this same script (two rocprofv3
+# --pmc passes, FETCH_SIZE and WRITE_SIZE, scaled by what the counters read for a 1 GiB device copy); the file
+# is read at run time, so a kernel without a line there reports null instead of a stale figure.
+TRAFFIC_FILES = {"c1": "selattn_fwd_bwd_S65536_bf16_hbm_traffic_pmc.txt"}
+TRAFFIC_KERNEL_NAMES = {"selattn_bwd_dqdkdv": "attn_bwd_dkdv_kernel", "selattn_fwd_main": "selattn_fwd_main_kernel",
+                        "selattn_fwd_reduce": "selattn_fwd_reduce_kernel",
+                        "selattn_bwd_dq_reduce": "selattn_bwd_reduce_kernel",
+                        "selattn_bwd_delta": "selattn_bwd_delta_kernel"}
+
+
+def measured_traffic(workload: str):
+    """{(label, gqa): bytes per launch} from profiles/<summary>: lines `<kernel> grid=<n> gqa=<g> ... bytes=<x> GB`."""
+    import re
+    out = {}
+    path = os.path.join(ROOT, "profiles", TRAFFIC_FILES.get(workload, "-"))
+    if not os.path.exists(path):
+        return out
+    for line in open(path):
+        m = re.match(r"^(\S+)\s+grid=\s*\d+\s+gqa=(\d+)\s.*bytes=([0-9.]+) GB", line)
+        if not m:
+            continue
+        for label, frag in TRAFFIC_KERNEL_NAMES.items():
+            if frag in m.group(1):
+                out[(label, int(m.group(2)))] = int(float(m.group(3)) * 1e9)
+    return out
 
 METRIC = "selected-attn fwd+bwd ms & TFLOP/s at 64K, B_K=64, T=16, GQA 1-4; roofline %"
 
@@ -58,35 +76,67 @@ def parse():
     return ap.parse_args()
 
 
-def cpu_baseline(seq_len: int, d: int, bk: int, topk: int, hkv: int):
-    """The CPU oracle (a PyTorch-eager port of the reference's math) timed on the host cores:
-    forward + backward of the same operator on a bounded sample of the workload."""
+def cpu_baseline(d: int, bk: int, topk: int, hkv: int, c1_seq_len: int, c1_p_key_per_head: int, sample_seq_len: int):
+    """The CPU oracle (a PyTorch-eager port of the reference's math; the reference has no CPU path of its own)
+    timed on the host cores.  `value`: the CPU-plumbing configuration exactly - forward of one sequence S=4096,
+    Hkv=Hq=4, fp32, median of 3.  Beside it the headline workload by extrapolation: forward + backward at
+    S=sample_seq_len timed once, scaled linearly in the number of unmasked (query, key) pairs to S=c1_seq_len at
+    GQA 1 (the cost of selected attention is linear in those pairs); labelled as an extrapolation."""
+    import statistics
     import torch
     from synth_inputs import make_qkv, make_topk_idx
     from oracle import selattn as orc
 
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    cu = [0, seq_len]
-    q, k, v, do = make_qkv(seq_len, hkv, hkv, d, torch.float32, seed=0)
-    idx = make_topk_idx(cu, hkv, bk, topk, seed=1)
-    _, p_key = orc.count_pairs(idx, bk, cu)
-    flops = 14.0 * d * p_key  # summed over heads already (g = 1)
+    s0 = 4096
+    q, k, v = make_qkv(s0, hkv, hkv, d, torch.float32, seed=0, with_do=False)
+    idx = make_topk_idx([0, s0], hkv, bk, topk, seed=1)
+    _, p_key0 = orc.count_pairs(idx, bk, [0, s0])
     times = []
-    for _ in range(2):
+    for _ in range(3):
         t0 = time.perf_counter()
-        orc.selected_attention_grads_ref(q, k, v, idx, bk, cu, do)
+        orc.selected_attention_ref(q, k, v, idx, bk, [0, s0])
         times.append(time.perf_counter() - t0)
-    best = min(times)
-    return {
-        "value": flops / best / 1e12,
+    c0 = statistics.median(times)
+    out = {
+        "value": round(4.0 * d * p_key0 / c0 / 1e12, 5),
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"oracle fwd+bwd (fp32 eager PyTorch), 1 sequence S={seq_len}, Hkv=Hq={hkv}, D={d}, "
-                  f"B_K={bk}, T={topk}; best of 2 runs, {best * 1e3:.0f} ms",
-        "ms": best * 1e3,
+        "sample": f"oracle forward (fp32 eager PyTorch), 1 sequence S={s0}, Hkv=Hq={hkv}, D={d}, B_K={bk}, "
+                  f"T={topk}: median of 3 runs {c0 * 1e3:.0f} ms",
+        "ms": round(c0 * 1e3, 1),
     }
+    s1 = sample_seq_len
+    q, k, v, do = make_qkv(s1, hkv, hkv, d, torch.float32, seed=0)
+    idx = make_topk_idx([0, s1], hkv, bk, topk, seed=1)
+    _, p_key1 = orc.count_pairs(idx, bk, [0, s1])
+    t0 = time.perf_counter()
+    orc.selected_attention_grads_ref(q, k, v, idx, bk, [0, s1], do)
+    t1 = time.perf_counter() - t0
+    factor = c1_p_key_per_head * hkv / p_key1
+    out["headline_extrapolated"] = {
+        "note": f"EXTRAPOLATION: oracle forward+backward timed at S={s1} (GQA 1, {t1 * 1e3:.0f} ms, "
+                f"{14.0 * d * p_key1 / t1 / 1e12:.4f} TFLOP/s), scaled by the ratio of unmasked (query, key) pairs "
+                f"({factor:.2f}) to S={c1_seq_len} at GQA 1",
+        "sample_ms": round(t1 * 1e3, 1),
+        "gqa1_fwd_bwd_ms": round(t1 * factor * 1e3, 0),
+    }
+    return out
+
+
+def _roofline_fields(name, ms, flops, nbytes):
+    """Roofline entry of one kernel: against the MFMA peak for the contraction kernels, against HBM otherwise."""
+    tf, gbs = flops / (ms * 1e-3) / 1e12, nbytes / (ms * 1e-3) / 1e9
+    if name in MFMA_KERNELS:
+        rec = dict(bound="mfma", achieved=round(tf, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
+                   frac=round(tf / MFMA_PEAK_TFLOPS, 4))
+    else:
+        rec = dict(bound="hbm", achieved=round(gbs, 2), peak=HBM_PEAK_GBS, unit="GB/s",
+                   frac=round(gbs / HBM_PEAK_GBS, 4))
+    rec.update(algo_tflops=round(tf, 2), algo_gbs=round(gbs, 1), algo_bytes=int(nbytes))
+    return rec
 
 
 def _kernel_records(kern, algo):
@@ -97,15 +147,7 @@ def _kernel_records(kern, algo):
         rec = {"kernel": name, "ms": round(ms, 4)}
         ab = algo.get(name)
         if ab is not None and ms > 0:
-            fl, by = ab
-            tf, gbs = fl / (ms * 1e-3) / 1e12, by / (ms * 1e-3) / 1e9
-            if tf / MFMA_PEAK_TFLOPS > gbs / HBM_PEAK_GBS:
-                rec.update(bound="mfma", achieved=round(tf, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s",
-                           frac=round(tf / MFMA_PEAK_TFLOPS, 4))
-            else:
-                rec.update(bound="hbm", achieved=round(gbs, 2), peak=HBM_PEAK_GBS, unit="GB/s",
-                           frac=round(gbs / HBM_PEAK_GBS, 4))
-            rec.update(algo_tflops=round(tf, 2), algo_gbs=round(gbs, 1))
+            rec.update(_roofline_fields(name, ms, ab[0], ab[1]))
         out.append(rec)
     return out
 
@@ -332,50 +374,59 @@ def main():
     kv_once = 2 * n * hkv * d * e          # K and V (or dK and dV) of every kv head, once
 
     def algo(name, g):
-        """(flops, bytes) one launch must do at the least: MFMA flops over unmasked (query, key) pairs,
-        HBM bytes of the tensors it has to read and write once."""
+        """(flops, least bytes, gather-model bytes) of one launch.  flops: MFMA work over the unmasked (query, key)
+        pairs.  least bytes: every input and output tensor once, plus the partial rows that the two-stage design
+        writes in one kernel and reads in the next, plus the index lists.  gather-model bytes: the same with q / dO
+        rows counted once per (query, block) pair, i.e. what the block-major kernels request when no gathered row
+        is found in a cache - the distance between the two is the re-gather of query rows."""
         hq = hkv * g
         pg = pairs * g                      # (query, head, block) rows
-        if name == "selattn_fwd_main":      # S = QK^T, O = PV; Q row in, normalised partial row + lse out
-            return 4.0 * d * p_key * g, pg * (2 * d * e + 4) + kv_once
-        if name == "selattn_bwd_dqdkdv":    # S, dP, dV, dK, dQ; Q, dO rows in, dQ partial row out, lse + delta in
-            return 10.0 * d * p_key * g, pg * (3 * d * e + 8) + 2 * kv_once
-        if name == "selattn_bwd_dq":
-            return 6.0 * d * p_key * g, pg * (3 * d * e + 8) + kv_once
-        if name == "selattn_bwd_dkdv":
-            return 8.0 * d * p_key * g, pg * (2 * d * e + 8) + 2 * kv_once
+        q_once = n * hq * d * e
+        idx_lists = 4 * pairs + 8 * nblk * hkv
+        if name == "selattn_fwd_main":      # S = QK^T, O = PV; q in, normalised partial row + lse out
+            least = q_once + kv_once + pg * (d * e + 4) + idx_lists
+            return 4.0 * d * p_key * g, least, least - q_once + pg * d * e
+        if name == "selattn_bwd_dqdkdv":    # S, dP, dV, dK, dQ; q, dO, lse, delta, k, v in; dQ partial rows, dk, dv out
+            least = 2 * q_once + 8 * n * hq + 2 * kv_once + pg * d * e + idx_lists
+            return 10.0 * d * p_key * g, least, least - 2 * q_once - 8 * n * hq + pg * (2 * d * e + 8)
         if name == "selattn_fwd_reduce":
-            return 0.0, pg * (d * e + 4) + n * hq * (d * e + 4)
+            by = pg * (d * e + 4) + n * hq * (d * e + 4) + 4 * hkv * n * topk
+            return 0.0, by, by
         if name == "selattn_bwd_dq_reduce":
-            return 0.0, pg * d * e + n * hq * d * e
+            by = pg * d * e + q_once + 4 * hkv * n * topk
+            return 0.0, by, by
         if name == "selattn_bwd_delta":
-            return 0.0, 2 * n * hq * d * e + n * hq * 4
+            by = 2 * q_once + n * hq * 4
+            return 0.0, by, by
         if name == "index_build":
-            return 0.0, 4 * hkv * n * topk * 2 + 4 * (pairs + 2 * nblk * hkv)
-        # selattn_bwd_dkdv_reduce: no least work of its own - dK / dV written once are counted in the fused
-        # kernel; it only adds up the fp32 partials of blocks that were split over several work-groups
-        return 0.0, 0.0
+            by = 4 * hkv * n * topk * 2 + 4 * (pairs + 2 * nblk * hkv)
+            return 0.0, by, by
+        return 0.0, 0.0, 0.0
 
+    traffic_of = measured_traffic(args.workload) if (n, d, bk, topk) == (65536, 128, 64, 16) else {}
     kernels = []
     for (name, g), ms in sorted(kern.items(), key=lambda kv: -kv[1]):
-        fl, by = algo(name, g)
-        tf, gbs = fl / (ms * 1e-3) / 1e12, by / (ms * 1e-3) / 1e9
-        f_mfma, f_hbm = tf / MFMA_PEAK_TFLOPS, gbs / HBM_PEAK_GBS
+        fl, by, by_gather = algo(name, g)
         rec = {"kernel": name, "gqa": g, "ms": round(ms, 4)}
         if fl == 0 and by == 0:
             kernels.append(rec)
             continue
-        if f_mfma > f_hbm:                  # the roofline that binds is the one the kernel sits closer to
-            rec.update(bound="mfma", achieved=round(tf, 2), peak=MFMA_PEAK_TFLOPS, unit="TFLOP/s", frac=round(f_mfma, 4))
-        else:
-            rec.update(bound="hbm", achieved=round(gbs, 2), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(f_hbm, 4))
-        rec.update(algo_tflops=round(tf, 2), algo_gbs=round(gbs, 1), algo_bytes=int(by))
+        rec.update(_roofline_fields(name, ms, fl, by))
+        if name in MFMA_KERNELS:            # the HBM view beside the MFMA fraction, with both byte counts
+            rec["hbm"] = {"least_bytes": int(by), "frac_least": round(by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                          "gather_model_bytes": int(by_gather),
+                          "frac_gather_model": round(by_gather / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+        tr = traffic_of.get((name, g))
+        rec["traffic"] = tr
+        if tr:
+            rec["traffic_over_least"] = round(tr / by, 2)
         kernels.append(rec)
     dom = kernels[0]
-    traffic = PMC_TRAFFIC_BYTES.get((dom["kernel"], dom["gqa"])) if (n, d, bk, topk) == (65536, 128, 64, 16) else None
     roofline = {"kernel": f"{dom['kernel']} (GQA {dom['gqa']})", "bound": dom["bound"],
                 "achieved": dom["achieved"], "peak": dom["peak"], "unit": dom["unit"], "frac": dom["frac"],
-                "traffic": traffic}
+                "traffic": dom.get("traffic")}
+    if "hbm" in dom:
+        roofline["hbm"] = dom["hbm"]
 
     per_gqa = []
     for g in groups:
@@ -411,7 +462,27 @@ def main():
         "kernels": kernels,
     }
     if not args.no_cpu_baseline and args.workload == "c1":
-        out["cpu_baseline"] = cpu_baseline(args.cpu_seq_len, d, bk, topk, hkv)
+        out["cpu_baseline"] = cpu_baseline(d, bk, topk, hkv, n, p_key // hkv, args.cpu_seq_len)
+        # the same shape on the GPU, for the speed-up at equal work
+        s0 = 4096
+        q0, k0, v0 = (x.to(dev) for x in make_qkv(s0, hkv, hkv, d, dtype, seed=0, with_do=False))
+        cu0 = torch.tensor([0, s0], dtype=torch.int32, device=dev)
+        idx0 = make_topk_idx([0, s0], hkv, bk, topk, seed=1).to(dev)
+        for _ in range(3):
+            _topk_sparse_attention_fwd_opt(q0, k0, v0, idx0, bk, cu0, cu0, s0, s0, scale)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            _topk_sparse_attention_fwd_opt(q0, k0, v0, idx0, bk, cu0, cu0, s0, s0, scale)
+        torch.cuda.synchronize()
+        gpu0 = (time.perf_counter() - t0) * 1e3 / 20
+        out["cpu_baseline"]["gpu_ms_same_shape"] = round(gpu0, 4)
+        out["cpu_baseline"]["speedup_same_shape"] = round(out["cpu_baseline"]["ms"] / gpu0, 1)
+        g1 = [r for r in per_gqa if r["gqa"] == 1]
+        if g1:
+            gpu1 = g1[0]["index_ms"] + g1[0]["fwd_ms"] + g1[0]["bwd_ms"]
+            out["cpu_baseline"]["headline_extrapolated"]["speedup_gqa1"] = round(
+                out["cpu_baseline"]["headline_extrapolated"]["gqa1_fwd_bwd_ms"] / gpu1, 0)
     print(json.dumps(out))
 
 

@@ -378,6 +378,7 @@ struct DecTopkParams {
   int batch, hkv, g;
   int kernel_size, kernel_stride, block_size, topk, init_blocks, local_blocks;
   int as_written;
+  int scores_to_bf16;      // rank the block scores after rounding them to bf16 (what the prefill selection does)
   float scale_log2;
   int32_t* topk_idx;       // [Hkv, B, topk]
   float* block_score;      // optional [Hkv, B, score_ld]
@@ -416,7 +417,7 @@ decode_topk_kernel(DecTopkParams p) {
       }
     }
     if (blk < p.init_blocks || (bq >= blk && bq < blk + p.local_blocks)) acc = INFINITY;
-    bs[blk] = acc;
+    bs[blk] = p.scores_to_bf16 ? (float)(__bf16)acc : acc;
     if (p.block_score) p.block_score[((int64_t)h * p.batch + b) * p.score_ld + blk] = acc;
   }
   if (p.block_score)
@@ -607,8 +608,8 @@ extern "C" int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const flo
                                int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
                                int32_t kernel_size, int32_t kernel_stride, int32_t block_size,
                                int32_t topk, int32_t init_blocks, int32_t local_blocks,
-                               int32_t as_written, float softmax_scale, int64_t max_blocks,
-                               int32_t* topk_idx, float* block_score, void* stream_) {
+                               int32_t as_written, int32_t scores_to_bf16, float softmax_scale,
+                               int64_t max_blocks, int32_t* topk_idx, float* block_score, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   FSA_CHECK_ARG(raw_score && lse && cu_ck && pos && seqlens && topk_idx, "fsa_decode_topk: null pointer");
   FSA_CHECK_ARG(batch >= 1 && topk >= 1 && num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
@@ -622,6 +623,7 @@ extern "C" int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const flo
   p.batch = batch; p.hkv = num_kv_heads; p.g = num_q_heads / num_kv_heads;
   p.kernel_size = kernel_size; p.kernel_stride = kernel_stride; p.block_size = block_size; p.topk = topk;
   p.init_blocks = init_blocks; p.local_blocks = local_blocks; p.as_written = as_written;
+  p.scores_to_bf16 = scores_to_bf16;
   p.scale_log2 = softmax_scale * LOG2E; p.topk_idx = topk_idx; p.block_score = block_score;
   p.score_ld = max_blocks;
   {

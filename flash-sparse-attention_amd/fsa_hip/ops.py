@@ -284,8 +284,9 @@ def decode_cmpattn(q, ck, cv, cu_ck, pos, kernel_size, kernel_stride, max_ck, so
 
 def decode_topk(raw_score, lse, cu_ck, pos, seqlens, num_q_heads, kernel_size, kernel_stride, block_size,
                 topk, max_blocks, init_blocks=1, local_blocks=2, softmax_scale=1.0, as_written=False,
-                return_block_score=False):
-    """Top-k block ids [Hkv,B,topk] int32 (descending score) for the decode step."""
+                return_block_score=False, scores_to_bf16=False):
+    """Top-k block ids [Hkv,B,topk] int32 (descending score) for the decode step; scores_to_bf16 ranks the block
+    scores after rounding them to bf16 (what the prefill selection of the layer does)."""
     _require_cuda(raw_score, lse, cu_ck, pos, seqlens)
     lib = _lib.load()
     hkv, b, ld = raw_score.shape
@@ -294,7 +295,8 @@ def decode_topk(raw_score, lse, cu_ck, pos, seqlens, num_q_heads, kernel_size, k
     bscore = torch.empty((hkv, b, max_blocks), dtype=torch.float32, device=dev) if return_block_score else None
     rc = lib.fsa_decode_topk(_ptr(raw_score), ld, _ptr(lse), _ptr(cu_ck), _ptr(pos), _ptr(seqlens), b,
                              num_q_heads, hkv, kernel_size, kernel_stride, block_size, topk, init_blocks,
-                             local_blocks, 1 if as_written else 0, float(softmax_scale), int(max_blocks),
+                             local_blocks, 1 if as_written else 0, 1 if scores_to_bf16 else 0,
+                             float(softmax_scale), int(max_blocks),
                              _ptr(idx), _ptr(bscore), _stream(dev))
     _lib.check(rc, "fsa_decode_topk")
     return (idx, bscore) if return_block_score else idx

@@ -5,7 +5,9 @@ The reference handles exactly one request (it asserts a single query row); so do
 the batched entry points live in fsa_hip.ops.decode_cmpattn / decode_topk.  `as_written=True`
 reproduces the reference's block-score conventions literally (candidate blocks counted from the
 compressed length, own block taken as 0, kv head h scored by q-head h); the default scores what
-prefill scores for the last token.  The returned ids are ordered by descending score."""
+prefill scores for the last token, and ranks the block scores after rounding them to bf16 as the
+prefill layer does (scores_to_bf16; the reference's decode ranks fp32 scores, which as_written
+keeps).  The returned ids are ordered by descending score."""
 import math
 import warnings
 from typing import Tuple
@@ -32,6 +34,7 @@ def _compressed_attention_decode(
     local_blocks: int = 2,
     query_start_index: int = 0,
     as_written: bool = False,
+    scores_to_bf16: bool = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     assert q.dtype == torch.bfloat16 or q.dtype == torch.float16
     assert q.dtype == k.dtype and k.dtype == v.dtype
@@ -54,5 +57,6 @@ def _compressed_attention_decode(
     nblk = max(nblk, 1)
     seqlens = torch.tensor([seqlen], dtype=torch.int32, device=dev)
     idx = _ops.decode_topk(raw, lse, cu_seqlens_k, pos, seqlens, q.shape[1], kernel_size, kernel_stride, block_size,
-                           min(topk, nblk), nblk, init_blocks, local_blocks, sm_scale, as_written=as_written)
+                           min(topk, nblk), nblk, init_blocks, local_blocks, sm_scale, as_written=as_written,
+                           scores_to_bf16=(not as_written) if scores_to_bf16 is None else scores_to_bf16)
     return o, idx  # idx: [num_kv_heads, 1, min(topk, nblk)] int32

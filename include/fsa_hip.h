@@ -241,7 +241,11 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
  * than topk blocks exist.  as_written = 1 reproduces the reference literally
  * (candidate blocks = ceil(compressed_len / block_size), own block taken as 0);
  * as_written = 0 uses ceil(seqlens[b] / block_size) blocks and own block
- * (seqlens[b]-1) / block_size.  block_score is optional [Hkv, B, max_blocks].
+ * (seqlens[b]-1) / block_size.  scores_to_bf16 != 0 ranks the block scores after
+ * rounding them to bf16, as the prefill selection of the layer does
+ * (nsa_ref/ops/compressed_attention.py:1307-1308), so that a decode step picks the
+ * blocks the prefill picks for the same token; the reference's decode ranks fp32
+ * scores (0).  block_score is optional [Hkv, B, max_blocks] (fp32, unrounded).
  *
  * fsa_decode_selattn replaces _topk_sparse_attention_decode
  * (fsa_preview/ops/selected_attention_decode.py:8-42): the g heads of a group
@@ -276,8 +280,8 @@ int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const float* lse, co
                     const int32_t* pos, const int32_t* seqlens, int32_t batch, int32_t num_q_heads,
                     int32_t num_kv_heads, int32_t kernel_size, int32_t kernel_stride, int32_t block_size,
                     int32_t topk, int32_t init_blocks, int32_t local_blocks, int32_t as_written,
-                    float softmax_scale, int64_t max_blocks, int32_t* topk_idx, float* block_score,
-                    void* stream);
+                    int32_t scores_to_bf16, float softmax_scale, int64_t max_blocks, int32_t* topk_idx,
+                    float* block_score, void* stream);
 
 int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
                        int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,

@@ -39,7 +39,7 @@ def test_decode_step_equals_prefill_last_token(dev, L):
     cv_full, _ = linear_compress(v, wk, cu, ks, st, None)
     # compressed attention + selection for the last token
     o_p, idx_p = compressed_attention(q, ck_full, cv_full, ks, st, bk, t, cu, cu_ck, L, n_full, None, 1, 2,
-                                      parallel_topk_compute=True)   # fp32 scores, as the decode path uses
+                                      parallel_topk_compute=False)  # bf16-rounded scores, the layer's path
     cu_q1 = torch.tensor([0, 1], dtype=torch.int32, device=dev)
     o_d, idx_d = _compressed_attention_decode(q[L - 1:], ck_full, cv_full, ks, st, bk, t, cu_q1, cu_ck, 1, n_full,
                                               None, 1, 2, query_start_index=L - 1)

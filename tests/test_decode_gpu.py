@@ -84,6 +84,10 @@ def test_decode_compressed_and_topk(dev, lens, hq, hkv, d, bk, t, dtype, as_writ
     # selection bit-exact given the kernel's block scores
     bscore, idx = bscore.cpu(), idx.cpu()
     assert torch.equal(idx, orc.decode_topk_ref(bscore, t))
+    # ... and with the scores rounded to bf16 before ranking (the prefill layer's rule; -inf slots stay -inf)
+    idx16 = ops.decode_topk(raw, lse, cu_ck_t, pos.to(dev), seqlens.to(dev), hq, KS, ST, bk, t, nblk_max,
+                            softmax_scale=1.0 / math.sqrt(d), as_written=as_written, scores_to_bf16=True)
+    assert torch.equal(idx16.cpu(), orc.decode_topk_ref(bscore.to(torch.bfloat16).float(), t))
     # block scores vs the oracle
     bs_r = orc.decode_block_scores_ref(q.float(), ck.float(), lse_r, cu_ck, pos, lens, KS, ST, bk,
                                        as_written=as_written, nblk_cols=nblk_max)
