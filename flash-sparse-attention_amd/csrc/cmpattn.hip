@@ -589,15 +589,19 @@ __device__ __forceinline__ float round_bf16(float x) { return (float)(__bf16)x; 
 // is packed with its id into one sortable 32-bit key - bf16 bits above, 0xFFFF - id below, so that the larger
 // key is the larger score or, on equal scores, the lower id - and lives in a register; a selection round is a
 // plain unsigned maximum over the wave.  NREG == 0: fp32 scores in LDS, (value, id) compared explicitly.
-template <int NREG>
-__global__ void __launch_bounds__(256)
+// BIG (more than 64 selected blocks per query, or more blocks than four waves can keep in LDS): one wave per
+// work-group, the chosen ids are collected in LDS behind the scores and ranked from there.
+template <int NREG, bool BIG = false>
+__global__ void __launch_bounds__(BIG ? 64 : 256)
 cmp_topk_kernel(TopkParams p) {
-  extern __shared__ float bs_all[];  // [4 waves][nblk], NREG == 0 only
+  constexpr int WPB = BIG ? 1 : 4;   // waves (= queries) per work-group
+  extern __shared__ float bs_all[];  // [WPB waves][nblk] (+ [t_out] ids when BIG), NREG == 0 only
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const int h = blockIdx.y;
-  const int tok = blockIdx.x * 4 + wv;  // the same for every lane of the wave
+  const int tok = blockIdx.x * WPB + wv;  // the same for every lane of the wave
   if (tok >= p.n_tokens) return;
   float* bs = bs_all + wv * p.nblk;
+  int* sel = reinterpret_cast<int*>(bs_all + p.nblk);  // BIG only
   const int s = upper_seg(p.cu_q, p.batch, tok);
   const int qi = tok - p.cu_q[s];
   const int nc = p.cu_k[s + 1] - p.cu_k[s];
@@ -679,10 +683,22 @@ cmp_topk_kernel(TopkParams p) {
       const uint64_t mine = best < 0.f ? 0ull : ((uint64_t)__float_as_uint(best) << 32) | (0xFFFFFFFFu - (uint32_t)best_id);
       const uint64_t top = wave_max_u64(mine);
       best_id = (int)(0xFFFFFFFFu - (uint32_t)top);
-      if (lane == t) my_id = best_id;
-      if (lane == 0) bs[best_id] = -1.f;
+      if (!BIG && lane == t) my_id = best_id;
+      if (lane == 0) {
+        bs[best_id] = -1.f;
+        if (BIG) sel[t] = best_id;
+      }
       __builtin_amdgcn_wave_barrier();
     }
+  }
+  if (BIG) {  // ascending order by rank counting over the list in LDS, then the mask
+    for (int i = lane; i < p.t_out; i += 64) {
+      const int id = sel[i];
+      int rank = 0;
+      for (int j = 0; j < p.t_out; ++j) rank += sel[j] < id;
+      p.topk_idx[((int64_t)h * p.n_tokens + tok) * p.t_out + rank] = id > bq ? -1 : id;
+    }
+    return;
   }
   // ascending order by rank counting (ids are distinct), then mask ids above the own block
   const int t_eff = min(p.t_out, 64);
@@ -979,8 +995,11 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   FSA_CHECK_ARG(topk >= 1 && max_seqlen_q >= 1 && max_seqlen_k >= 1, "fsa_cmp_topk: bad sizes");
   const int nblk = (int)((max_seqlen_q + block_size - 1) / block_size);
   const int t_out = topk < nblk ? topk : nblk;
-  FSA_CHECK_ARG(t_out <= 64, "fsa_cmp_topk: at most 64 blocks can be selected per query");
-  FSA_CHECK_ARG(nblk * 16 <= 64 * 1024, "fsa_cmp_topk: more than 4096 selection blocks per sequence");
+  // more than 64 selected blocks per query or more than 4096 blocks per sequence: one-wave work-groups with
+  // scores and chosen ids in LDS, which bounds their sum
+  const bool big = t_out > 64 || nblk > 4096;
+  FSA_CHECK_ARG(!big || ((int64_t)nblk + t_out) * 4 <= 160 * 1024,
+                "fsa_cmp_topk: blocks per sequence + selected blocks per query exceed 40960");
   // usual geometry (window of 2 strides, block of 4): the score kernel writes block scores, at most
   // max_seqlen_k / 4 + 1 per query, instead of one probability per compressed key
   const bool rebin = kernel_size == 2 * kernel_stride && block_size == 4 * kernel_stride;
@@ -1012,7 +1031,12 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   {
     ProfScope ps_("cmp_topk", stream);
     const dim3 grid((unsigned)((total_q + 3) / 4), (unsigned)num_kv_heads);
-    if (scores_to_bf16 && nblk <= 128) cmp_topk_kernel<2><<<grid, 256, 0, stream>>>(tp);
+    if (big) {
+      const int lds = (nblk + t_out) * 4;
+      rc = cmp_set_lds(cmp_topk_kernel<0, true>, lds);
+      if (rc) return rc;
+      cmp_topk_kernel<0, true><<<dim3((unsigned)total_q, (unsigned)num_kv_heads), 64, lds, stream>>>(tp);
+    } else if (scores_to_bf16 && nblk <= 128) cmp_topk_kernel<2><<<grid, 256, 0, stream>>>(tp);
     else if (scores_to_bf16 && nblk <= 256) cmp_topk_kernel<4><<<grid, 256, 0, stream>>>(tp);
     else if (scores_to_bf16 && nblk <= 512) cmp_topk_kernel<8><<<grid, 256, 0, stream>>>(tp);
     else if (scores_to_bf16 && nblk <= 1024) cmp_topk_kernel<16><<<grid, 256, 0, stream>>>(tp);

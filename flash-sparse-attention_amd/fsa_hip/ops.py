@@ -24,6 +24,30 @@ def _stream(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+# Head dims the kernels are built for.  Any other head_dim <= 256 (the reference accepts every head_dim <= 256,
+# README.md:63, by padding tiles to the next power of two inside its kernels) runs on the next built size with
+# zero-padded rows: q.k and P.V are unchanged by zero columns, the softmax scale is taken from the true head_dim,
+# and the padded columns of the outputs and gradients are cut off again.
+_NATIVE_D = (64, 128, 256)
+
+
+def _native_dim(d: int, native=_NATIVE_D) -> int:
+    for nd in native:
+        if d <= nd:
+            return nd
+    raise ValueError(f"head_dim {d} is not supported (at most {native[-1]})")
+
+
+def _pad_d(t: Optional[torch.Tensor], d_to: int):
+    if t is None or t.shape[-1] == d_to:
+        return t
+    return torch.nn.functional.pad(t, (0, d_to - t.shape[-1]))
+
+
+def _cut_d(t: torch.Tensor, d: int):
+    return t[..., :d].contiguous()
+
+
 def _require_cuda(*tensors):
     for t in tensors:
         if not t.is_cuda:
@@ -109,6 +133,10 @@ def selattn_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, index: SelInd
     assert hkv == index.num_kv_heads and n == index.total_tokens
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        o, lse = selattn_fwd(_pad_d(q, dn), _pad_d(k, dn), _pad_d(v, dn), index, softmax_scale)
+        return _cut_d(o, d), lse
     dev = q.device
     o = torch.empty((n, hq, d), dtype=q.dtype, device=dev)
     lse = torch.empty((hq, n), dtype=torch.float32, device=dev)
@@ -137,6 +165,11 @@ def selattn_bwd(q, k, v, o, do, lse, index: SelIndex, softmax_scale: Optional[fl
     hkv = k.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        g = selattn_bwd(_pad_d(q, dn), _pad_d(k, dn), _pad_d(v, dn), _pad_d(o, dn), _pad_d(do, dn), lse, index,
+                        softmax_scale)
+        return tuple(_cut_d(t, d) for t in g)
     if do.stride(2) != 1:
         do = do.contiguous()
     if o.stride(2) != 1:
@@ -178,6 +211,11 @@ def cmpattn_fwd(q, ck, cv, kernel_size, kernel_stride, cu_q, cu_k, max_seqlen_q,
     hkv = ck.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        o, lse = cmpattn_fwd(_pad_d(q, dn), _pad_d(ck, dn), _pad_d(cv, dn), kernel_size, kernel_stride, cu_q, cu_k,
+                             max_seqlen_q, softmax_scale)
+        return _cut_d(o, d), lse
     o = torch.empty_like(q)
     lse = torch.empty((hq, n), dtype=torch.float32, device=q.device)
     if ck.shape[0] == 0:
@@ -200,6 +238,11 @@ def cmpattn_bwd(q, ck, cv, o, do, lse, kernel_size, kernel_stride, cu_q, cu_k, m
     nk, hkv, _ = ck.shape
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        g = cmpattn_bwd(_pad_d(q, dn), _pad_d(ck, dn), _pad_d(cv, dn), _pad_d(o, dn), _pad_d(do, dn), lse, kernel_size,
+                        kernel_stride, cu_q, cu_k, max_seqlen_q, softmax_scale)
+        return tuple(_cut_d(t, d) for t in g)
     if do.stride(2) != 1:
         do = do.contiguous()
     dq = torch.empty((n, hq, d), dtype=q.dtype, device=q.device)
@@ -230,6 +273,11 @@ def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_
     hkv = ck.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        return cmp_topk(_pad_d(q, dn), _pad_d(ck, dn), lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_k,
+                        max_seqlen_q, max_seqlen_k, init_blocks, local_blocks, softmax_scale, scores_to_bf16,
+                        return_block_score)
     nblk = (int(max_seqlen_q) + block_size - 1) // block_size
     t_out = min(topk, nblk)
     dev = q.device
@@ -265,6 +313,11 @@ def decode_cmpattn(q, ck, cv, cu_ck, pos, kernel_size, kernel_stride, max_ck, so
     hkv = ck.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        o, lse, raw = decode_cmpattn(_pad_d(q, dn), _pad_d(ck, dn), _pad_d(cv, dn), cu_ck, pos, kernel_size,
+                                     kernel_stride, max_ck, softmax_scale, want_scores, score_head_as_written)
+        return _cut_d(o, d), lse, raw
     dev = q.device
     o = torch.empty((b, hq, d), dtype=q.dtype, device=dev)
     lse = torch.empty((hq, b), dtype=torch.float32, device=dev)
@@ -314,6 +367,11 @@ def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scal
     assert topk_idx.shape[0] == hkv and topk_idx.shape[1] == b
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        o, lse = decode_selattn(_pad_d(q, dn), _pad_d(k_cache, dn), _pad_d(v_cache, dn), cu_k, topk_idx, block_size,
+                                softmax_scale)
+        return _cut_d(o, d), lse
     dev = q.device
     o = torch.empty((b, hq, d), dtype=q.dtype, device=dev)
     lse = torch.empty((hq, b), dtype=torch.float32, device=dev)
@@ -361,6 +419,10 @@ def winattn_fwd(q, k, v, cu_seqlens, max_seqlen, window, softmax_scale=None):
     hkv = k.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        o, lse = winattn_fwd(_pad_d(q, dn), _pad_d(k, dn), _pad_d(v, dn), cu_seqlens, max_seqlen, window, softmax_scale)
+        return _cut_d(o, d), lse
     o = torch.empty((n, hq, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((hq, n), dtype=torch.float32, device=q.device)
     rc = lib.fsa_winattn_fwd(_ptr(q), _ptr(k), _ptr(v), _DTYPE[q.dtype], q.stride(0), q.stride(1), k.stride(0),
@@ -379,6 +441,11 @@ def winattn_bwd(q, k, v, o, do, lse, cu_seqlens, max_seqlen, window, softmax_sca
     hkv = k.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(d)
+    dn = _native_dim(d)
+    if dn != d:
+        g = winattn_bwd(_pad_d(q, dn), _pad_d(k, dn), _pad_d(v, dn), _pad_d(o, dn), _pad_d(do, dn), lse, cu_seqlens,
+                        max_seqlen, window, softmax_scale)
+        return tuple(_cut_d(t, d) for t in g)
     if do.stride(2) != 1:
         do = do.contiguous()
     dev = q.device
@@ -412,12 +479,24 @@ def rope(x, cu_seqlens, inv_freq, attention_scaling=1.0, start=0, stride=1, inve
     return out
 
 
+def _pad_compress_weight(w, kernel_size: int, d: int, dn: int):
+    """w [H, ks*d, d] as [H, ks*dn, dn] with zero rows / columns for the padded dims."""
+    h = w.shape[0]
+    w4 = torch.nn.functional.pad(w.view(h, kernel_size, d, d), (0, dn - d, 0, dn - d))
+    return w4.reshape(h, kernel_size * dn, dn).contiguous()
+
+
 def linear_compress_fwd(x, w, cu_x, cu_y, total_y, max_y, kernel_size, kernel_stride, pe=None):
     """y [total_y, H, D] = strided-window projection of x [N, H, D] with w [H, ks*D, D] (+ pe bias)."""
     _require_cuda(x, w, cu_x, cu_y)
     assert x.dtype in _DTYPE and x.dtype == w.dtype and x.stride(2) == 1 and w.is_contiguous()
     lib = _lib.load()
     n, h, d = x.shape
+    dn = _native_dim(d)
+    if dn != d:
+        y = linear_compress_fwd(_pad_d(x, dn), _pad_compress_weight(w, kernel_size, d, dn), cu_x, cu_y, total_y, max_y,
+                                kernel_size, kernel_stride, None if pe is None else _pad_d(pe, dn).contiguous())
+        return _cut_d(y, d)
     y = torch.empty((int(total_y), h, d), dtype=x.dtype, device=x.device)
     bias = torch.empty((h, d), dtype=x.dtype, device=x.device) if pe is not None else None
     if pe is not None:
@@ -435,6 +514,13 @@ def linear_compress_bwd(x, w, dy, cu_x, cu_y, max_x, kernel_size, kernel_stride,
     _require_cuda(x, w, dy, cu_x, cu_y)
     lib = _lib.load()
     n, h, d = x.shape
+    dn = _native_dim(d, (128, 256))   # the weight-gradient kernel works on 128 input dims per work-group
+    if dn != d:
+        dx, dw, dpe = linear_compress_bwd(_pad_d(x, dn), _pad_compress_weight(w, kernel_size, d, dn), _pad_d(dy, dn),
+                                          cu_x, cu_y, max_x, kernel_size, kernel_stride,
+                                          None if pe is None else _pad_d(pe, dn).contiguous())
+        dw = dw.view(h, kernel_size, dn, dn)[:, :, :d, :d].reshape(h, kernel_size * d, d).contiguous()
+        return _cut_d(dx, d), dw, (None if dpe is None else _cut_d(dpe, d))
     dev = x.device
     dy = dy.contiguous()
     dx = torch.empty((n, h, d), dtype=x.dtype, device=dev)

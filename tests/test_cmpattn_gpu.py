@@ -133,13 +133,19 @@ TOPK_VARIANTS = [
     ([0, 40, 20040], 32, 24, True),      # 625 blocks, a sequence shorter than one block
     ([0, 5000], 64, 16, False),          # fp32 scores
     ([0, 17000], 16, 16, True),          # 1063 blocks
+    # beyond what a wave keeps in registers / four waves keep in LDS: one wave per work-group, ids ranked from LDS
+    ([0, 300, 7000], 64, 80, True),      # 80 selected blocks per query (the first sequence has 5)
+    ([0, 66000], 16, 8, False, 1),       # 4125 blocks
 ]
 
 
-@pytest.mark.parametrize("cu,bk,t,to_bf16", TOPK_VARIANTS)
-def test_cmp_topk_variants(dev, cu, bk, t, to_bf16):
+@pytest.mark.parametrize("case", TOPK_VARIANTS)
+def test_cmp_topk_variants(dev, case):
+    cu, bk, t, to_bf16 = case[:4]
     print(f"case cu={cu} bk={bk} t={t} to_bf16={to_bf16}", flush=True)
     hq, hkv, d, ks, st, dtype = 2, 2, 64, 32, 16, torch.bfloat16
+    if len(case) > 4:
+        hq = hkv = case[4]
     q, ck, cv, do, cu_k = _make(cu, hq, hkv, d, ks, st, dtype, seed=13)
     cu_q_t = torch.tensor(cu, dtype=torch.int32, device=dev)
     cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)

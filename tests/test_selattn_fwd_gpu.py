@@ -58,6 +58,10 @@ CASES = [
     ([0, 900], 2, 2, 64, 128, 4, torch.float16),
     ([0, 500], 4, 2, 256, 32, 6, torch.float16),
     ([0, 700], 2, 1, 256, 64, 6, torch.bfloat16),
+    # head dims without a kernel of their own run zero-padded on the next size up (the reference takes any <= 256)
+    ([0, 800], 4, 2, 96, 64, 8, torch.bfloat16),
+    ([0, 600], 2, 1, 40, 32, 4, torch.float16),
+    ([0, 500], 2, 2, 192, 64, 4, torch.bfloat16),
 ]
 
 
