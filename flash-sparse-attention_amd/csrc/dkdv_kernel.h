@@ -28,6 +28,7 @@ struct SelBwdParams {
   const int32_t* starts;
   const int32_t* sel_tokens;
   const int32_t* tile_prefix;
+  const int32_t* tile_block;  // [Hkv, max_tiles]: block of every tile, or null (binary search through tile_prefix)
   int batch;
   int64_t max_blocks;
   int64_t cap;
@@ -186,7 +187,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
   const int32_t* tp = p.tile_prefix + h * nbp1;
   const int w = blockIdx.x;
   if (w >= tp[p.max_blocks]) return;
-  const int gb = upper_seg(tp, (int)p.max_blocks, w);
+  const int gb = p.tile_block ? p.tile_block[h * p.max_tiles + w] : upper_seg(tp, (int)p.max_blocks, w);
   KvBlock<MODE, BK> blk;
   blk.init(p, gb);
   const int rows = p.counts[h * p.max_blocks + gb] * p.g;

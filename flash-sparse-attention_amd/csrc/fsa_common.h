@@ -237,4 +237,8 @@ struct ProfScope {
 
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
+// fsa_build_tiles with an optional tile -> block table [num_kv_heads, max_tiles] (max_tiles >= fsa_max_tiles(...))
+int build_tiles(const int32_t* counts, int num_kv_heads, int64_t max_blocks, int group_size, int rows_per_tile,
+                int32_t* tile_prefix, int32_t* tile_block, int64_t max_tiles, hipStream_t stream);
+
 }  // namespace fsa

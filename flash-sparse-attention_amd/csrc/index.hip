@@ -414,7 +414,7 @@ split_blocks_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int6
 
 __global__ void __launch_bounds__(SCAN_THREADS)
 tiles_kernel(const int32_t* __restrict__ counts, int64_t max_blocks, int group_size, int rows_per_tile,
-             int32_t* __restrict__ tile_prefix) {
+             int32_t* __restrict__ tile_prefix, int32_t* __restrict__ tile_block, int64_t max_tiles) {
   const int h = blockIdx.x;
   const int32_t* c = counts + h * max_blocks;
   int32_t* tp = tile_prefix + h * (max_blocks + 1);
@@ -430,7 +430,11 @@ tiles_kernel(const int32_t* __restrict__ counts, int64_t max_blocks, int group_s
   int run = block_exclusive_scan(sum, &total);
   for (int64_t i = lo; i < hi; ++i) {
     tp[i] = run;
-    run += ntile(i);
+    const int nt = ntile(i);
+    // tile -> block, so that a work-group finds its block with one load instead of a binary search through tp
+    if (tile_block)
+      for (int t = 0; t < nt; ++t) tile_block[h * max_tiles + run + t] = (int32_t)i;
+    run += nt;
   }
   if (threadIdx.x == 0) tp[max_blocks] = total;
 }
@@ -591,16 +595,23 @@ extern "C" int fsa_split_topk_blocks(const int32_t* topk_idx, int64_t topk_strid
   return 0;
 }
 
-extern "C" int fsa_build_tiles(const int32_t* counts, int32_t num_kv_heads, int64_t max_blocks,
-                               int32_t group_size, int32_t rows_per_tile, int32_t* tile_prefix,
-                               void* stream_) {
+int fsa::build_tiles(const int32_t* counts, int num_kv_heads, int64_t max_blocks, int group_size,
+                     int rows_per_tile, int32_t* tile_prefix, int32_t* tile_block, int64_t max_tiles,
+                     hipStream_t stream) {
   FSA_CHECK_ARG(counts && tile_prefix, "fsa_build_tiles: null pointer");
   FSA_CHECK_ARG(num_kv_heads >= 1 && max_blocks >= 1 && group_size >= 1 && rows_per_tile >= 1,
                 "fsa_build_tiles: sizes must be positive");
-  tiles_kernel<<<num_kv_heads, SCAN_THREADS, 0, (hipStream_t)stream_>>>(counts, max_blocks, group_size,
-                                                                        rows_per_tile, tile_prefix);
+  tiles_kernel<<<num_kv_heads, SCAN_THREADS, 0, stream>>>(counts, max_blocks, group_size, rows_per_tile,
+                                                          tile_prefix, tile_block, max_tiles);
   FSA_CHECK_LAUNCH("fsa_build_tiles");
   return 0;
+}
+
+extern "C" int fsa_build_tiles(const int32_t* counts, int32_t num_kv_heads, int64_t max_blocks,
+                               int32_t group_size, int32_t rows_per_tile, int32_t* tile_prefix,
+                               void* stream_) {
+  return fsa::build_tiles(counts, num_kv_heads, max_blocks, group_size, rows_per_tile, tile_prefix, nullptr, 0,
+                          (hipStream_t)stream_);
 }
 
 extern "C" int64_t fsa_max_tiles(int64_t total_tokens, int32_t topk, int32_t group_size,

@@ -107,7 +107,7 @@ selattn_bwd_reduce_kernel(SelBwdParams p, DqReduceArgs a, int n_kv, int hkv) {
 
 // ------------------------------------------------------------- host side ----
 struct BwdWs {
-  size_t off_delta, off_dqpart, off_tiles_kv, off_kvpart, total;
+  size_t off_delta, off_dqpart, off_tiles_kv, off_tile_block, off_kvpart, total;
   int64_t max_tiles_kv;
 };
 
@@ -119,7 +119,8 @@ static BwdWs bwd_ws_layout(int64_t n, int hq, int hkv, int d, int topk, int bk, 
   w.off_delta = 0;
   w.off_dqpart = align_up((size_t)n * hq * 4, 256);
   w.off_tiles_kv = w.off_dqpart + align_up(cap * hkv * g * d * 2, 256);
-  w.off_kvpart = w.off_tiles_kv + align_up((size_t)hkv * (max_blocks + 1) * 4, 256);
+  w.off_tile_block = w.off_tiles_kv + align_up((size_t)hkv * (max_blocks + 1) * 4, 256);
+  w.off_kvpart = w.off_tile_block + align_up((size_t)hkv * w.max_tiles_kv * 4, 256);
   w.total = w.off_kvpart + align_up((size_t)hkv * w.max_tiles_kv * 2 * bk * d * 4, 256);
   return w;
 }
@@ -239,7 +240,9 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   char* wsp = (char*)workspace;
   float* delta = (float*)(wsp + ws.off_delta);
   int32_t* tiles_kv = (int32_t*)(wsp + ws.off_tiles_kv);
-  int rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, kv_tile_rows(g, head_dim, block_size), tiles_kv, stream_);
+  int32_t* tile_block = (int32_t*)(wsp + ws.off_tile_block);
+  int rc = build_tiles(counts, num_kv_heads, max_blocks, g, kv_tile_rows(g, head_dim, block_size), tiles_kv, tile_block,
+                       ws.max_tiles_kv, stream);
   if (rc) return rc;
 
   const int64_t cap = total_tokens * topk;
@@ -264,7 +267,7 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   p.dk = dk; p.dv = dv;
   p.dk_sn = (int64_t)num_kv_heads * head_dim; p.dk_sh = head_dim;
   p.cu_seqlens_k = nullptr; p.kernel_size = 0; p.kernel_stride = 1;
-  p.tile_prefix = tiles_kv; p.max_tiles = ws.max_tiles_kv; p.kv_tile_rows = kv_tile_rows(g, head_dim, block_size);
+  p.tile_prefix = tiles_kv; p.tile_block = tile_block; p.max_tiles = ws.max_tiles_kv; p.kv_tile_rows = kv_tile_rows(g, head_dim, block_size);
 
   DqReduceArgs red;
   red.dq_part = p.dq_part; red.slot_of = slot_of; red.cap = cap; red.n_tokens = total_tokens;

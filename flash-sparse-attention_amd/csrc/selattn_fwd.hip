@@ -28,6 +28,8 @@ struct SelFwdParams {
   const int32_t* starts;
   const int32_t* sel_tokens;
   const int32_t* tile_prefix;
+  const int32_t* tile_block;  // [Hkv, max_tiles]: block of every tile
+  int64_t max_tiles;
   int batch;
   int64_t max_blocks;
   int64_t cap;  // N * T: capacity of the per-head pair list
@@ -95,7 +97,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   const int32_t* tp = p.tile_prefix + h * nbp1;
   const int w = blockIdx.x;
   if (w >= tp[p.max_blocks]) return;
-  const int gb = upper_seg(tp, (int)p.max_blocks, w);
+  const int gb = p.tile_block[h * p.max_tiles + w];
   const int s = upper_seg(p.cu_blocks, p.batch, gb);
   const int b_local = gb - p.cu_blocks[s];
   const int seq_start = p.cu_seqlens[s], seq_end = p.cu_seqlens[s + 1];
@@ -381,17 +383,21 @@ selattn_fwd_reduce_kernel(const T* __restrict__ o_part, const float* __restrict_
 }
 
 struct FwdWs {
-  size_t off_opart, off_lse, off_tiles, total;
+  size_t off_opart, off_lse, off_tiles, off_tile_block, total;
+  int64_t max_tiles;
 };
 
-static FwdWs fwd_ws_layout(int64_t n_tokens, int hq, int hkv, int d, int topk, int64_t max_blocks) {
+// bk <= 0: the block size is not known (workspace query): room for the smallest tiles any block size uses
+static FwdWs fwd_ws_layout(int64_t n_tokens, int hq, int hkv, int d, int topk, int bk, int64_t max_blocks) {
   FwdWs w;
   const int g = hq / hkv;
   const size_t cap = (size_t)n_tokens * topk;
   w.off_opart = 0;
   w.off_lse = align_up(cap * hkv * g * d * 2, 256);
   w.off_tiles = w.off_lse + align_up(cap * hkv * g * 4, 256);
-  w.total = w.off_tiles + align_up((size_t)hkv * (max_blocks + 1) * 4, 256);
+  w.off_tile_block = w.off_tiles + align_up((size_t)hkv * (max_blocks + 1) * 4, 256);
+  w.max_tiles = fsa_max_tiles(n_tokens, topk, g, bk > 0 ? sel_tile_rows(g, d, bk) : 1024, max_blocks);
+  w.total = w.off_tile_block + align_up((size_t)hkv * fsa_max_tiles(n_tokens, topk, g, 1024, max_blocks) * 4, 256);
   return w;
 }
 
@@ -462,7 +468,7 @@ using namespace fsa;
 extern "C" size_t fsa_selattn_fwd_workspace_bytes(int64_t total_tokens, int32_t num_q_heads,
                                                   int32_t num_kv_heads, int32_t head_dim, int32_t topk,
                                                   int64_t max_blocks) {
-  return fwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, max_blocks).total;
+  return fwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, 0, max_blocks).total;
 }
 
 extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int32_t dtype,
@@ -492,16 +498,18 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
   FSA_CHECK_ARG(q_stride_n >= 0 && q_stride_n < ((int64_t)1 << 31) && q_stride_h >= 0 &&
                     g * q_stride_h + head_dim < ((int64_t)1 << 31),
                 "fsa_selattn_fwd: q strides too large or negative");
-  FwdWs ws = fwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, max_blocks);
+  FwdWs ws = fwd_ws_layout(total_tokens, num_q_heads, num_kv_heads, head_dim, topk, block_size, max_blocks);
   if (!workspace || workspace_bytes < ws.total) {
     set_error("fsa_selattn_fwd: workspace too small (%zu < %zu)", workspace_bytes, ws.total);
     return FSA_ERR_WORKSPACE;
   }
   char* wsp = (char*)workspace;
   int32_t* tile_prefix = (int32_t*)(wsp + ws.off_tiles);
-  int rc = fsa_build_tiles(counts, num_kv_heads, max_blocks, g, sel_tile_rows(g, head_dim, block_size), tile_prefix, stream_);
+  int32_t* tile_block = (int32_t*)(wsp + ws.off_tile_block);
+  const int64_t max_tiles = ws.max_tiles;
+  int rc = build_tiles(counts, num_kv_heads, max_blocks, g, sel_tile_rows(g, head_dim, block_size), tile_prefix,
+                       tile_block, max_tiles, stream);
   if (rc) return rc;
-  const int64_t max_tiles = fsa_max_tiles(total_tokens, topk, g, sel_tile_rows(g, head_dim, block_size), max_blocks);
 
   SelFwdParams p;
   p.q = q; p.k = k; p.v = v;
@@ -509,7 +517,7 @@ extern "C" int fsa_selattn_fwd(const void* q, const void* k, const void* v, int3
   p.k_sn = k_stride_n; p.k_sh = k_stride_h;
   p.v_sn = v_stride_n; p.v_sh = v_stride_h;
   p.cu_seqlens = cu_seqlens; p.cu_blocks = cu_blocks; p.counts = counts; p.starts = starts;
-  p.sel_tokens = sel_tokens; p.tile_prefix = tile_prefix;
+  p.sel_tokens = sel_tokens; p.tile_prefix = tile_prefix; p.tile_block = tile_block; p.max_tiles = max_tiles;
   p.batch = batch; p.max_blocks = max_blocks; p.cap = total_tokens * topk; p.g = g;
   p.g_shift = group_shift(g);
 
