@@ -119,9 +119,21 @@ def test_cmp_topk(dev, cu, hq, hkv, d, ks, st, bk, t, dtype):
     assert (diff <= 2.0 ** -6 * bs_r[~inf_r].abs() + 2e-3).all()   # no tap lost anywhere
     # 3. against the oracle end to end: rows whose k-th and (k+1)-th scores differ clearly must match
     want_e2e = orc.topk_select_ref(bs_r, t, cu, bk, to_bf16=False)
-    same = (idx == want_e2e).all(-1).float().mean().item()
-    print(f"  rows identical to the oracle's end-to-end selection: {same:.4f}", flush=True)
-    assert same > 0.9
+    same_rows = (idx == want_e2e).all(-1)
+    same = same_rows.float().mean().item()
+    # tie rate: rows whose k-th and (k+1)-th bf16 scores are EQUAL (the set depends on the tie rule), and rows where
+    # the two are closer than the kernel's and the oracle's scores may differ (last-place differences before the
+    # bf16 rounding move either score to the neighbouring value).  Every row outside the second group must agree.
+    tie = orc.kth_value_tie_rows(bs_r, t, to_bf16=False)
+    srt = torch.sort(bs_r, dim=-1, descending=True).values
+    kth, nxt = srt[..., min(t, srt.shape[-1]) - 1], srt[..., min(t, srt.shape[-1] - 1)]
+    near = (kth - nxt) <= 2 * (2.0 ** -6 * kth.abs() + 2e-3)   # twice the bound asserted on a single score above
+    near |= torch.isinf(kth) & torch.isinf(nxt)
+    print(f"  rows identical to the oracle's end-to-end selection: {same:.4f}; tie rate {tie.float().mean().item():.4f}, "
+          f"closer than the score bound {near.float().mean().item():.4f}; differing rows outside them: "
+          f"{(~same_rows & ~near).sum().item()}", flush=True)
+    assert (same_rows | near).all()
+    assert same > 0.999
 
 
 # one case per variant of the selection kernel: block scores in 4 / 8 / 16 registers per lane (rounded to bf16),
