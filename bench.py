@@ -206,7 +206,7 @@ def side_workload(args):
             "selattn_fwd_reduce": (0.0, rows * (d * e + 4) + n * hq * (d * e + 4)),
             "selattn_bwd_dqdkdv": (10.0 * d * p_key * g, rows * (3 * d * e + 8) + 2 * kvbytes),
             "selattn_bwd_dq_reduce": (0.0, rows * d * e + qbytes),
-            "selattn_bwd_delta": (0.0, 2 * qbytes + 4 * n * hq),
+            "selattn_bwd_delta": (0.0, 2 * qbytes + 12 * n * hq),   # o, dO, lse in; (lse, delta) pairs out
             "cmpattn_bwd_delta": (0.0, 2 * qbytes + 4 * n * hq),
             "winattn_bwd_delta": (0.0, 2 * qbytes + 4 * n * hq),
             "cmpattn_fwd": (4.0 * d * vis_c * hq, 2 * qbytes + ckv),
@@ -396,7 +396,7 @@ def main():
             by = pg * d * e + q_once + 4 * hkv * n * topk
             return 0.0, by, by
         if name == "selattn_bwd_delta":
-            by = 2 * q_once + n * hq * 4
+            by = 2 * q_once + n * hq * 12    # o, dO, lse in; (lse, delta) pairs out
             return 0.0, by, by
         if name == "index_build":
             by = 4 * hkv * n * topk * 2 + 4 * (pairs + 2 * nblk * hkv)

@@ -21,6 +21,10 @@ struct SelBwdParams {
   const void* d_o;
   const float* lse;    // [Hq, N]
   const float* delta;  // [Hq, N]
+  // selected mode: (lse, delta) pairs [N, Hq] instead of the two arrays above - the rows of a block are scattered
+  // queries, and the statistics of a query's g heads then share one 8 g byte piece of a line instead of 2 g lines
+  const float2* stat2;
+  int hq;              // q heads in all (selected mode)
   int64_t q_sn, q_sh, k_sn, k_sh, v_sn, v_sh, do_sn, do_sh;
   const int32_t* cu_seqlens;
   const int32_t* cu_blocks;
@@ -287,9 +291,15 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         const int trank = div_group(r, p.g, p.g_shift), head = r - trank * p.g;
         const int token = tok_stat;
         // token ids are 32-bit, so n_tokens < 2^31: one 32 x 32 -> 64 bit multiply-add
-        const uint64_t stat = (uint64_t)(uint32_t)(h * p.g + head) * (uint32_t)p.n_tokens + (uint32_t)token;
-        lse_st = p.lse[stat];
-        del_st = p.delta[stat];
+        if (MODE == KV_MODE_SELECTED) {
+          const float2 s2 = p.stat2[(uint64_t)(uint32_t)token * (uint32_t)p.hq + (uint32_t)(h * p.g + head)];
+          lse_st = s2.x;
+          del_st = s2.y;
+        } else {
+          const uint64_t stat = (uint64_t)(uint32_t)(h * p.g + head) * (uint32_t)p.n_tokens + (uint32_t)token;
+          lse_st = p.lse[stat];
+          del_st = p.delta[stat];
+        }
         lim_st = blk.limit(p, token - blk.seq_start);
         llo_st = blk.limit_lo(p, token - blk.seq_start);
       }

@@ -1,6 +1,6 @@
 // Selected attention backward for gfx950.
 //
-//   delta    : delta[h, n] = sum_d O * dO                       (HBM stream)
+//   delta    : (lse, sum_d O * dO) pairs [N, Hq]                (HBM stream)
 //   dqdkdv   : block-major, contraction over the gathered rows (dkdv_kernel.h
 //              with FUSE_DQ).  Each wave owns 16 keys of the block and keeps
 //              their K / V fragments in registers; Q / dO tiles of 64 rows go
@@ -26,7 +26,7 @@ template <typename T, int D>
 __global__ void __launch_bounds__(256)
 selattn_bwd_delta_kernel(const T* __restrict__ o, int64_t o_sn, int64_t o_sh,
                          const T* __restrict__ d_o, int64_t do_sn, int64_t do_sh, int64_t n_tokens,
-                         int hq, float* __restrict__ delta) {
+                         int hq, const float* __restrict__ lse, float2* __restrict__ stat2) {
   typedef typename Elem<T>::vec8 vec8;
   constexpr int LPR = D / 8, RPB = 256 / LPR;
   const int64_t R = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
@@ -41,7 +41,7 @@ selattn_bwd_delta_kernel(const T* __restrict__ o, int64_t o_sn, int64_t o_sh,
   for (int e = 0; e < 8; ++e) s += (float)a[e] * (float)b[e];
 #pragma unroll
   for (int o_ = LPR / 2; o_ >= 1; o_ >>= 1) s += __shfl_xor(s, o_, LPR);
-  if (sub == 0) delta[(int64_t)h * n_tokens + tok] = s;
+  if (sub == 0) stat2[R] = make_float2(lse[(int64_t)h * n_tokens + tok], s);  // [N, Hq] pairs
 }
 
 // Sum of the <= T partial dQ rows of each (query, head).
@@ -117,7 +117,7 @@ static BwdWs bwd_ws_layout(int64_t n, int hq, int hkv, int d, int topk, int bk, 
   const size_t cap = (size_t)n * topk;
   w.max_tiles_kv = fsa_max_tiles(n, topk, g, kv_tile_rows(g, d, bk), max_blocks);
   w.off_delta = 0;
-  w.off_dqpart = align_up((size_t)n * hq * 4, 256);
+  w.off_dqpart = align_up((size_t)n * hq * 8, 256);
   w.off_tiles_kv = w.off_dqpart + align_up(cap * hkv * g * d * 2, 256);
   w.off_tile_block = w.off_tiles_kv + align_up((size_t)hkv * (max_blocks + 1) * 4, 256);
   w.off_kvpart = w.off_tile_block + align_up((size_t)hkv * w.max_tiles_kv * 4, 256);
@@ -176,7 +176,7 @@ static int dispatch_bwd(int d, int bk, const SelBwdParams& pkv, int hkv, int64_t
 
 template <typename T>
 static int launch_delta(int d, const void* o, int64_t o_sn, int64_t o_sh, const void* d_o, int64_t do_sn,
-                        int64_t do_sh, int64_t n, int hq, float* delta, hipStream_t stream) {
+                        int64_t do_sh, int64_t n, int hq, const float* lse, float2* stat2, hipStream_t stream) {
   const int64_t rows = n * hq;
 #define FSA_CASE(DD)                                                                                     \
   if (d == DD) {                                                                                         \
@@ -184,7 +184,7 @@ static int launch_delta(int d, const void* o, int64_t o_sn, int64_t o_sh, const 
     const unsigned grid = (unsigned)((rows + RPB - 1) / RPB);                                            \
     ProfScope ps_("selattn_bwd_delta", stream);                                                          \
     selattn_bwd_delta_kernel<T, DD><<<grid, 256, 0, stream>>>((const T*)o, o_sn, o_sh, (const T*)d_o,    \
-                                                              do_sn, do_sh, n, hq, delta);               \
+                                                              do_sn, do_sh, n, hq, lse, stat2);          \
     return 0;                                                                                            \
   }
   FSA_CASE(64)
@@ -238,7 +238,7 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
     return FSA_ERR_WORKSPACE;
   }
   char* wsp = (char*)workspace;
-  float* delta = (float*)(wsp + ws.off_delta);
+  float2* stat2 = (float2*)(wsp + ws.off_delta);
   int32_t* tiles_kv = (int32_t*)(wsp + ws.off_tiles_kv);
   int32_t* tile_block = (int32_t*)(wsp + ws.off_tile_block);
   int rc = build_tiles(counts, num_kv_heads, max_blocks, g, kv_tile_rows(g, head_dim, block_size), tiles_kv, tile_block,
@@ -248,14 +248,14 @@ extern "C" int fsa_selattn_bwd(const void* q, const void* k, const void* v, cons
   const int64_t cap = total_tokens * topk;
   rc = dtype == FSA_BF16
            ? launch_delta<__bf16>(head_dim, o, o_stride_n, o_stride_h, d_o, do_stride_n, do_stride_h,
-                                  total_tokens, num_q_heads, delta, stream)
+                                  total_tokens, num_q_heads, lse, stat2, stream)
            : launch_delta<_Float16>(head_dim, o, o_stride_n, o_stride_h, d_o, do_stride_n, do_stride_h,
-                                    total_tokens, num_q_heads, delta, stream);
+                                    total_tokens, num_q_heads, lse, stat2, stream);
   if (rc) return rc;
   FSA_CHECK_LAUNCH("fsa_selattn_bwd delta");
 
   SelBwdParams p;
-  p.q = q; p.k = k; p.v = v; p.d_o = d_o; p.lse = lse; p.delta = delta;
+  p.q = q; p.k = k; p.v = v; p.d_o = d_o; p.lse = lse; p.delta = nullptr; p.stat2 = stat2; p.hq = num_q_heads;
   p.q_sn = q_stride_n; p.q_sh = q_stride_h; p.k_sn = k_stride_n; p.k_sh = k_stride_h;
   p.v_sn = v_stride_n; p.v_sh = v_stride_h; p.do_sn = do_stride_n; p.do_sh = do_stride_h;
   p.cu_seqlens = cu_seqlens; p.cu_blocks = cu_blocks; p.counts = counts; p.starts = starts;
