@@ -233,17 +233,77 @@ constexpr int CT_ITEMS = 4096;                       // entries per tile (a whol
 constexpr int CT_ROUNDS = CT_ITEMS / CT_THREADS;     // entries per thread
 constexpr int CT_MAX_BUCKETS = 4096;                 // max_blocks + 1 must not exceed this (LDS: 16 B per bucket)
 
-__device__ __forceinline__ int item_bucket(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
-                                           const int32_t* __restrict__ cu_seqlens,
-                                           const int32_t* __restrict__ cu_blocks, int batch, int h, int token,
-                                           int t, int sentinel) {
-  const int b = topk_idx[h * stride_h + (int64_t)token * stride_n + t];
-  const int s = upper_seg(cu_seqlens, batch, token);
-  const int b0 = cu_blocks[s], nb = cu_blocks[s + 1] - b0;
-  return (b >= 0 && b < nb) ? b0 + b : sentinel;
+// Sequences that the consecutive queries of a tile belong to.  Almost every tile lies inside one sequence: its
+// block range is then looked up once per work-group, and the bucket of an entry is its block id plus a constant -
+// the loads of all entries of a thread are independent and in flight together.  (A search per entry puts a chain of
+// dependent loads into every round.)
+struct SeqSpan {
+  int s_lo, s_hi;  // sequence of the first / last query
+  int b0, nb;      // first global block and block count of sequence s_lo
+};
+__device__ __forceinline__ SeqSpan seq_span(const int32_t* __restrict__ cu_seqlens,
+                                            const int32_t* __restrict__ cu_blocks, int batch, int tok_first,
+                                            int tok_last) {
+  SeqSpan sp;
+  sp.s_lo = upper_seg(cu_seqlens, batch, tok_first);
+  sp.s_hi = upper_seg(cu_seqlens, batch, tok_last);
+  sp.b0 = cu_blocks[sp.s_lo];
+  sp.nb = cu_blocks[sp.s_lo + 1] - sp.b0;
+  return sp;
 }
 
-// table[h][bucket][tile] = entries of the tile that fall into the bucket
+// i / d for 0 <= i < 2^22, d >= 1 with rcp = 1.0f / d: the float product is off by less than one, one correction
+// step makes it exact (a handful of instructions against some forty for the integer division)
+__device__ __forceinline__ int div_small(int i, int d, float rcp) {
+  int q = (int)((float)i * rcp);
+  const int r = i - q * d;
+  q += (r >= d ? 1 : 0) - (r < 0 ? 1 : 0);
+  return q;
+}
+
+// Block ids of CT_ROUNDS entries of a tile: entry numbers idx[r] (negative: none).  All loads are issued together,
+// without branches, and before anything that waits for another load.
+__device__ __forceinline__ void load_block_ids(const int32_t* __restrict__ topk_idx, int64_t stride_h,
+                                               int64_t stride_n, int h, int tok0, int topk, int n_it,
+                                               const int* idx, int* raw) {
+  const float rcp = 1.0f / (float)topk;
+  const int32_t* base = topk_idx + h * stride_h;
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r) {
+    const int i = min(max(idx[r], 0), n_it - 1);
+    const int qi = div_small(i, topk, rcp), t = i - qi * topk;
+    raw[r] = base[(int64_t)(tok0 + qi) * stride_n + t];
+  }
+}
+
+// block ids -> buckets (global block ids; `sentinel` for padding and out-of-range ids; -1 where there is no entry)
+__device__ __forceinline__ void ids_to_buckets(const int32_t* __restrict__ cu_seqlens,
+                                               const int32_t* __restrict__ cu_blocks, int batch, const SeqSpan& sp,
+                                               int tok0, int topk, int sentinel, const int* idx, const int* raw,
+                                               int* key) {
+  if (sp.s_lo == sp.s_hi) {  // uniform over the work-group
+#pragma unroll
+    for (int r = 0; r < CT_ROUNDS; ++r) {
+      const int b = raw[r];
+      key[r] = idx[r] < 0 ? -1 : (b >= 0 && b < sp.nb) ? sp.b0 + b : sentinel;
+    }
+  } else {
+    const float rcp = 1.0f / (float)topk;
+#pragma unroll
+    for (int r = 0; r < CT_ROUNDS; ++r) {
+      const int b = raw[r];  // raw and key may be the same array
+      int k = -1;
+      if (idx[r] >= 0) {
+        const int s = upper_seg(cu_seqlens, batch, tok0 + div_small(idx[r], topk, rcp));
+        const int b0 = cu_blocks[s], nb = cu_blocks[s + 1] - b0;
+        k = (b >= 0 && b < nb) ? b0 + b : sentinel;
+      }
+      key[r] = k;
+    }
+  }
+}
+
+// table[h][tile][bucket] = entries of the tile that fall into the bucket (a tile writes one contiguous row)
 __global__ void __launch_bounds__(CT_THREADS)
 count_tiles_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
                    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ cu_blocks, int batch,
@@ -251,77 +311,127 @@ count_tiles_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64
                    int32_t* __restrict__ table) {
   extern __shared__ int hist[];
   const int h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
-  for (int b = tid; b < nbuckets; b += CT_THREADS) hist[b] = 0;
-  __syncthreads();
   const int64_t tok0 = (int64_t)tile * q_per_tile;
   const int n_q = (int)min((int64_t)q_per_tile, n_tokens - tok0);
-  for (int i = tid; i < n_q * topk; i += CT_THREADS) {
-    const int qi = i / topk, t = i - qi * topk;
-    atomicAdd(&hist[item_bucket(topk_idx, stride_h, stride_n, cu_seqlens, cu_blocks, batch, h, (int)tok0 + qi, t,
-                                nbuckets - 1)], 1);
+  int key[CT_ROUNDS], idx[CT_ROUNDS];  // the tile has at most CT_ITEMS entries (host check)
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r) {
+    const int i = tid + r * CT_THREADS;
+    idx[r] = i < n_q * topk ? i : -1;
   }
+  load_block_ids(topk_idx, stride_h, stride_n, h, (int)tok0, topk, n_q * topk, idx, key);
+  for (int b = tid; b < nbuckets; b += CT_THREADS) hist[b] = 0;   // while the ids are on their way
   __syncthreads();
-  for (int b = tid; b < nbuckets; b += CT_THREADS) table[((int64_t)h * nbuckets + b) * ntiles + tile] = hist[b];
+  const SeqSpan sp = seq_span(cu_seqlens, cu_blocks, batch, (int)tok0, (int)tok0 + n_q - 1);
+  ids_to_buckets(cu_seqlens, cu_blocks, batch, sp, (int)tok0, topk, nbuckets - 1, idx, key, key);
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r)
+    if (key[r] >= 0) atomicAdd(&hist[key[r]], 1);
+  __syncthreads();
+  for (int b = tid; b < nbuckets; b += CT_THREADS) table[((int64_t)h * ntiles + tile) * nbuckets + b] = hist[b];
 }
 
-// one wave per (head, bucket): exclusive scan of its row of the table over the tiles; the row total is the
-// bucket's entry count
-__global__ void __launch_bounds__(CT_THREADS)
+// Exclusive scan of the table over the tiles, bucket by bucket; the total of a bucket is its entry count.  A
+// work-group takes 64 buckets (one per lane: the reads of a tile row are contiguous) and each of its waves an equal
+// share of the tiles: column sums of the shares, then the running prefix written back over the counts.
+constexpr int ST_WAVES = 16;
+__global__ void __launch_bounds__(ST_WAVES * WAVE)
 scan_tiles_kernel(int32_t* __restrict__ table, int ntiles, int nbuckets, int64_t max_blocks,
                   int32_t* __restrict__ counts, int32_t* __restrict__ bucket_total) {
-  const int h = blockIdx.y, lane = threadIdx.x & (WAVE - 1);
-  const int b = blockIdx.x * CT_WAVES + threadIdx.x / WAVE;
-  if (b >= nbuckets) return;
-  int32_t* row = table + ((int64_t)h * nbuckets + b) * ntiles;
-  int carry = 0;
-  for (int base = 0; base < ntiles; base += WAVE) {
-    const int i = base + lane;
-    const int v = i < ntiles ? row[i] : 0;
-    int inc = v;
-#pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) {
-      const int t = __shfl_up(inc, o, WAVE);
-      if (lane >= o) inc += t;
-    }
-    if (i < ntiles) row[i] = carry + inc - v;
-    carry += __shfl(inc, WAVE - 1, WAVE);
-  }
-  if (lane == 0) {
-    bucket_total[h * nbuckets + b] = carry;
-    if (b < max_blocks) counts[h * max_blocks + b] = carry;
-  }
-}
-
-// starts[h][0..max_blocks] = exclusive scan of the bucket totals (the padding bucket starts where the last
-// block ends)
-__global__ void __launch_bounds__(SCAN_THREADS)
-bucket_starts_kernel(const int32_t* __restrict__ bucket_total, int nbuckets, int32_t* __restrict__ starts) {
-  const int h = blockIdx.x;
-  const int32_t* c = bucket_total + h * nbuckets;
-  int32_t* st = starts + h * nbuckets;  // [Hkv, max_blocks + 1] with nbuckets = max_blocks + 1
-  const int per = (nbuckets + SCAN_THREADS - 1) / SCAN_THREADS;
-  const int lo = min(nbuckets, (int)threadIdx.x * per), hi = min(nbuckets, lo + per);
+  __shared__ int part[ST_WAVES][WAVE];
+  const int h = blockIdx.y, lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  const int b = blockIdx.x * WAVE + lane;
+  const bool live = b < nbuckets;
+  const int per = (ntiles + ST_WAVES - 1) / ST_WAVES;
+  const int t0 = min(ntiles, w * per), t1 = min(ntiles, t0 + per);
+  int32_t* col = table + (int64_t)h * ntiles * nbuckets + (live ? b : 0);
   int sum = 0;
-  for (int i = lo; i < hi; ++i) sum += c[i];
-  int total;
-  int run = block_exclusive_scan(sum, &total);
-  for (int i = lo; i < hi; ++i) {
-    st[i] = run;
-    run += c[i];
+  if (live) {
+#pragma unroll 8
+    for (int t = t0; t < t1; ++t) sum += col[(int64_t)t * nbuckets];
+  }
+  part[w][lane] = sum;
+  __syncthreads();
+  int run = 0;
+  for (int ww = 0; ww < w; ++ww) run += part[ww][lane];
+  if (live) {
+#pragma unroll 8
+    for (int t = t0; t < t1; ++t) {
+      const int v = col[(int64_t)t * nbuckets];
+      col[(int64_t)t * nbuckets] = run;
+      run += v;
+    }
+    if (w == ST_WAVES - 1) {  // the last share ends at the total
+      bucket_total[h * nbuckets + b] = run;
+      if (b < max_blocks) counts[h * max_blocks + b] = run;
+    }
   }
 }
 
+// Exclusive scans of two ints per thread over the CT_THREADS of a work-group.
+__device__ __forceinline__ void block_exclusive_scan2(int a, int b, int* ea, int* eb) {
+  __shared__ int wa[CT_WAVES], wb[CT_WAVES];
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  int ia = a, ib = b;
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const int ta = __shfl_up(ia, o, WAVE), tb = __shfl_up(ib, o, WAVE);
+    if (lane >= o) {
+      ia += ta;
+      ib += tb;
+    }
+  }
+  if (lane == WAVE - 1) {
+    wa[w] = ia;
+    wb[w] = ib;
+  }
+  __syncthreads();
+  int offa = 0, offb = 0;
+  for (int ww = 0; ww < w; ++ww) {
+    offa += wa[ww];
+    offb += wb[ww];
+  }
+  *ea = offa + ia - a;
+  *eb = offb + ib - b;
+  __syncthreads();
+}
+
+// LDS of place_items_kernel in ints: per-wave counters [CT_WAVES][nbuckets], reused as the list of positions of the
+// tile's sorted entries [CT_ITEMS]; per-bucket offset [nbuckets]; entry numbers of the sorted entries [CT_ITEMS] as
+// 16-bit values
+__host__ __device__ inline int place_lds_ints(int nbuckets) {
+  const int a = CT_WAVES * nbuckets > CT_ITEMS ? CT_WAVES * nbuckets : CT_ITEMS;
+  return a + nbuckets + CT_ITEMS / 2;
+}
+
+// Places the entries of one tile.  Position of an entry = start of its bucket (exclusive scan of the bucket totals,
+// done here by every work-group; tile 0 also stores it as `starts`) + entries of the bucket in earlier tiles (table)
+// + earlier entries of the bucket inside the tile.  The tile's entries are first put into bucket order in LDS, so
+// that neighbouring lanes store to neighbouring positions of `sel_tokens` (the few entries that a tile has in one
+// bucket are one store transaction instead of one each).
+// KEY_BITS: bits of a bucket id that the lanes of a wave are matched on (2^KEY_BITS >= nbuckets); a constant, so
+// that the matching below is straight-line code - as a loop over a run-time count it spends as much on the loop as
+// on the ballots.
+template <int KEY_BITS>
 __global__ void __launch_bounds__(CT_THREADS)
 place_items_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64_t stride_n,
                    const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ cu_blocks, int batch,
-                   int64_t n_tokens, int topk, int q_per_tile, int ntiles, int nbuckets, int key_bits,
-                   const int32_t* __restrict__ table, const int32_t* __restrict__ starts,
-                   int32_t* __restrict__ sel_tokens, int32_t* __restrict__ slot_of) {
-  extern __shared__ int cnt[];  // [CT_WAVES][nbuckets]
-  const int h = blockIdx.y, tile = blockIdx.x, tid = threadIdx.x;
+                   int64_t n_tokens, int topk, int q_per_tile, int ntiles, int nbuckets,
+                   const int32_t* __restrict__ table, const int32_t* __restrict__ bucket_total,
+                   int32_t* __restrict__ starts, int32_t* __restrict__ sel_tokens, int32_t* __restrict__ slot_of) {
+  extern __shared__ int lds[];
+  int* cnt = lds;                                  // [CT_WAVES][nbuckets]
+  int* sorted_pos = lds;                           // [CT_ITEMS], once the counters are no longer needed
+  int* delta = lds + max(CT_WAVES * nbuckets, CT_ITEMS);   // [nbuckets]: position in sel_tokens - position in the tile
+  uint16_t* sorted_item = reinterpret_cast<uint16_t*>(delta + nbuckets);  // [CT_ITEMS]
+  __shared__ int n_real_s;
+  // Work-groups go to the eight XCDs in turn, and each XCD has its own L2.  Consecutive tiles append to the same
+  // lines of sel_tokens: tiles are dealt so that an XCD gets a contiguous eighth of them (gridDim.x is a multiple
+  // of eight), and the pieces of a line meet in one L2 instead of leaving eight of them as partial lines.
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const int tile = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  if (tile >= ntiles) return;
   const int lane = tid & (WAVE - 1), w = tid / WAVE;
-  for (int i = tid; i < CT_WAVES * nbuckets; i += CT_THREADS) cnt[i] = 0;
-  __syncthreads();
   const int64_t tok0 = (int64_t)tile * q_per_tile;
   const int n_q = (int)min((int64_t)q_per_tile, n_tokens - tok0);
   const int n_it = n_q * topk;
@@ -332,30 +442,37 @@ place_items_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64
   const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   int* my_cnt = cnt + w * nbuckets;
   // all bucket ids first (the loads of every round in flight together), then the ordered ranking
+  {
+    int idx[CT_ROUNDS];
 #pragma unroll
-  for (int r = 0; r < CT_ROUNDS; ++r) {
-    key[r] = -1;
-    rank[r] = 0;
-    if (r < rounds) {  // uniform
+    for (int r = 0; r < CT_ROUNDS; ++r) {
       const int i = w * per_wave + r * WAVE + lane;
-      if (r * WAVE + lane < per_wave && i < n_it) {
-        const int qi = i / topk, t = i - qi * topk;
-        key[r] = item_bucket(topk_idx, stride_h, stride_n, cu_seqlens, cu_blocks, batch, h, (int)tok0 + qi, t,
-                             nbuckets - 1);
-      }
+      idx[r] = (r < rounds && r * WAVE + lane < per_wave && i < n_it) ? i : -1;
+      rank[r] = 0;
     }
+    load_block_ids(topk_idx, stride_h, stride_n, h, (int)tok0, topk, n_it, idx, key);
+    for (int i = tid; i < CT_WAVES * nbuckets; i += CT_THREADS) cnt[i] = 0;   // while the ids are on their way
+    __syncthreads();
+    const SeqSpan sp = seq_span(cu_seqlens, cu_blocks, batch, (int)tok0, (int)tok0 + n_q - 1);
+    ids_to_buckets(cu_seqlens, cu_blocks, batch, sp, (int)tok0, topk, nbuckets - 1, idx, key, key);
   }
 #pragma unroll
   for (int r = 0; r < CT_ROUNDS; ++r) {
     if (r < rounds) {  // uniform
       const bool ok = key[r] >= 0;
       const int kb = ok ? key[r] : 0;
-      uint64_t peers = __ballot(ok);
-      for (int bit = 0; bit < key_bits; ++bit) {
-        const bool one = (kb >> bit) & 1;
-        const uint64_t bb = __ballot(one);
-        peers &= one ? bb : ~bb;
+      const uint64_t valid = __ballot(ok);
+      uint32_t p_lo = (uint32_t)valid, p_hi = (uint32_t)(valid >> 32);
+#pragma unroll
+      for (int bit = 0; bit < KEY_BITS; ++bit) {
+        // lanes whose bit is set keep the lanes of the ballot, the others its complement: one sign-extending
+        // bit-field extract gives the XOR mask (0 or ~0) and the predicate of the ballot
+        const uint32_t flip = (uint32_t)__builtin_amdgcn_sbfe(~kb, bit, 1);
+        const uint64_t bb = __ballot(flip == 0u);
+        p_lo &= (uint32_t)bb ^ flip;
+        p_hi &= (uint32_t)(bb >> 32) ^ flip;
       }
+      const uint64_t peers = ((uint64_t)p_hi << 32) | p_lo;
       int old = 0;
       if (ok) {
         old = my_cnt[kb];
@@ -367,29 +484,78 @@ place_items_kernel(const int32_t* __restrict__ topk_idx, int64_t stride_h, int64
     }
   }
   __syncthreads();
-  // per bucket: first position of this tile's entries, then the exclusive prefix over the waves
-  for (int b = tid; b < nbuckets; b += CT_THREADS) {
-    int run = starts[h * nbuckets + b] + table[((int64_t)h * nbuckets + b) * ntiles + tile];
+  // Thread t finishes buckets [t * per, (t + 1) * per): two exclusive scans over the buckets - of the bucket totals
+  // (start of the bucket in sel_tokens) and of the tile's own counts (start of the bucket in the sorted tile).
+  constexpr int BPT = CT_MAX_BUCKETS / CT_THREADS;
+  const int per = (nbuckets + CT_THREADS - 1) / CT_THREADS;   // <= BPT
+  const int32_t* tot = bucket_total + h * nbuckets;
+  const int32_t* trow = table + ((int64_t)h * ntiles + tile) * nbuckets;
+  int tot_r[BPT], tab_r[BPT];
+  int sum_tot = 0, sum_tile = 0;
 #pragma unroll
-    for (int ww = 0; ww < CT_WAVES; ++ww) {
-      const int c = cnt[ww * nbuckets + b];
-      cnt[ww * nbuckets + b] = run;
-      run += c;
+  for (int j = 0; j < BPT; ++j) {
+    const int b = tid * per + j;
+    tot_r[j] = 0;
+    tab_r[j] = 0;
+    if (j < per && b < nbuckets) {
+      tot_r[j] = tot[b];
+      tab_r[j] = trow[b];
+      sum_tot += tot_r[j];
+#pragma unroll
+      for (int ww = 0; ww < CT_WAVES; ++ww) sum_tile += cnt[ww * nbuckets + b];
+    }
+  }
+  int g_run, l_run;
+  block_exclusive_scan2(sum_tot, sum_tile, &g_run, &l_run);
+#pragma unroll
+  for (int j = 0; j < BPT; ++j) {
+    const int b = tid * per + j;
+    if (j < per && b < nbuckets) {
+      if (tile == 0) starts[h * nbuckets + b] = g_run;   // [Hkv, max_blocks + 1] with nbuckets = max_blocks + 1
+      delta[b] = g_run + tab_r[j] - l_run;
+      if (b == nbuckets - 1) n_real_s = l_run;            // the padding bucket is the last one
+#pragma unroll
+      for (int ww = 0; ww < CT_WAVES; ++ww) {
+        const int c = cnt[ww * nbuckets + b];
+        cnt[ww * nbuckets + b] = l_run;
+        l_run += c;
+      }
+      g_run += tot_r[j];
     }
   }
   __syncthreads();
   const int64_t n_items = n_tokens * topk;
   int32_t* st = sel_tokens + h * n_items;
   int32_t* so = slot_of + h * n_items;
+  const int n_real = n_real_s;
+  // position in the sorted tile (kept in key[]) and in sel_tokens (rank[]); slot_of in entry order
 #pragma unroll
   for (int r = 0; r < CT_ROUNDS; ++r) {
     if (r < rounds && key[r] >= 0) {
       const int i = w * per_wave + r * WAVE + lane;
-      const int pos = my_cnt[key[r]] + rank[r];
-      const bool real = key[r] != nbuckets - 1;
-      st[pos] = real ? (int32_t)(tok0 + i / topk) : -1;
-      so[tok0 * topk + i] = real ? pos : -1;
+      const int lpos = my_cnt[key[r]] + rank[r];
+      const int pos = lpos + delta[key[r]];
+      so[tok0 * topk + i] = key[r] != nbuckets - 1 ? pos : -1;
+      key[r] = lpos;
+      rank[r] = pos;
+    } else {
+      key[r] = -1;
     }
+  }
+  __syncthreads();  // the counters are dead: their memory becomes the position list
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r) {
+    if (key[r] >= 0) {
+      sorted_pos[key[r]] = rank[r];
+      sorted_item[key[r]] = (uint16_t)(w * per_wave + r * WAVE + lane);
+    }
+  }
+  __syncthreads();
+  const float rcp = 1.0f / (float)topk;
+#pragma unroll
+  for (int r = 0; r < CT_ROUNDS; ++r) {
+    const int j = tid + r * CT_THREADS;
+    if (j < n_it) st[sorted_pos[j]] = j < n_real ? (int32_t)(tok0 + div_small((int)sorted_item[j], topk, rcp)) : -1;
   }
 }
 
@@ -522,23 +688,33 @@ extern "C" int fsa_build_index(const int32_t* topk_idx, int64_t topk_stride_h, i
     count_tiles_kernel<<<g_tiles, CT_THREADS, (size_t)c.nbuckets * 4, stream>>>(
         topk_idx, topk_stride_h, topk_stride_n, cu_seqlens, cu_blocks, batch, total_tokens, topk, c.q_per_tile,
         c.ntiles, c.nbuckets, table);
-    scan_tiles_kernel<<<dim3((c.nbuckets + CT_WAVES - 1) / CT_WAVES, num_kv_heads), CT_THREADS, 0, stream>>>(
+    scan_tiles_kernel<<<dim3((c.nbuckets + WAVE - 1) / WAVE, num_kv_heads), ST_WAVES * WAVE, 0, stream>>>(
         table, c.ntiles, c.nbuckets, max_blocks, counts, totals);
-    bucket_starts_kernel<<<num_kv_heads, SCAN_THREADS, 0, stream>>>(totals, c.nbuckets, starts);
-    const size_t lds = (size_t)CT_WAVES * c.nbuckets * 4;
-    static bool attr_done = false;
-    if (!attr_done && lds > 48 * 1024) {
-      hipError_t e = hipFuncSetAttribute((const void*)place_items_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, CT_WAVES * CT_MAX_BUCKETS * 4);
-      if (e != hipSuccess) {
-        set_error("hipFuncSetAttribute(place_items_kernel): %s", hipGetErrorString(e));
-        return (int)e;
-      }
-      attr_done = true;
-    }
-    place_items_kernel<<<g_tiles, CT_THREADS, lds, stream>>>(
-        topk_idx, topk_stride_h, topk_stride_n, cu_seqlens, cu_blocks, batch, total_tokens, topk, c.q_per_tile,
-        c.ntiles, c.nbuckets, key_bits, table, starts, sel_tokens, slot_of);
+    const size_t lds = (size_t)place_lds_ints(c.nbuckets) * 4;
+    dim3 g_place((c.ntiles + 7) / 8 * 8, num_kv_heads);
+#define FSA_PLACE(KB)                                                                                            \
+  {                                                                                                              \
+    static bool attr_done = false;                                                                               \
+    if (!attr_done && lds > 48 * 1024) {                                                                         \
+      hipError_t e = hipFuncSetAttribute((const void*)place_items_kernel<KB>,                                    \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,                     \
+                                         place_lds_ints(CT_MAX_BUCKETS) * 4);                                    \
+      if (e != hipSuccess) {                                                                                     \
+        set_error("hipFuncSetAttribute(place_items_kernel): %s", hipGetErrorString(e));                          \
+        return (int)e;                                                                                           \
+      }                                                                                                          \
+      attr_done = true;                                                                                          \
+    }                                                                                                            \
+    place_items_kernel<KB><<<g_place, CT_THREADS, lds, stream>>>(                                                \
+        topk_idx, topk_stride_h, topk_stride_n, cu_seqlens, cu_blocks, batch, total_tokens, topk, c.q_per_tile,  \
+        c.ntiles, c.nbuckets, table, totals, starts, sel_tokens, slot_of);                                       \
+  }
+    if (key_bits <= 7) FSA_PLACE(7)
+    else if (key_bits <= 9) FSA_PLACE(9)
+    else if (key_bits <= 10) FSA_PLACE(10)
+    else if (key_bits <= 11) FSA_PLACE(11)
+    else FSA_PLACE(12)
+#undef FSA_PLACE
     FSA_CHECK_LAUNCH("fsa_build_index");
     return 0;
   }
