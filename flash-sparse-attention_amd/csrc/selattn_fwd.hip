@@ -165,25 +165,28 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   };
   constexpr bool STAGED = SelLds<D, BK>::STAGE_OUT;  // false: LDS cannot hold the wave tiles, direct loads / stores
   vec8 qst[NLD];
+  // Direct mode: the Q fragments of a lane's row in the MFMA operand layout, straight from global memory.  k-step ks
+  // contracts dims [16 ks, 16 ks + 16): the two lanes of a row read 32 contiguous bytes and a cache line is used up
+  // by four consecutive loads.  Like qst they are requested one sub-tile ahead: as soon as the S^T products have
+  // consumed them, while the softmax and the O^T products of the current sub-tile run.
+  vec8 qdir[STAGED ? 1 : NKS];
+  auto fetch_dir = [&](int token, int sub_) {
+    const int rc_ = min(sub_ + col, row_hi - 1);
+    const uint32_t head_ = (uint32_t)(rc_ - div_group(rc_, p.g, p.g_shift) * p.g);
+    const T* qrow = qbase_row + ((uint64_t)(uint32_t)token * q_sn32 + (head_ * q_sh32 + hh * 8));
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) qdir[STAGED ? 0 : ks] = load16<vec8>(qrow + ks * 16);
+  };
   // one sub-tile: rows sub.. of the block; qst holds its Q rows (row-coalesced layout) on entry
   // and those of the next sub-tile (token ids tok_next) on exit
   auto step = [&](int token, int sub, int tok_next) {
     const int r = sub + col;
     const bool valid = r < row_hi;
-    vec8 qdir[STAGED ? 1 : NKS];
     if (STAGED) {
 #pragma unroll
       for (int j = 0; j < NLD; ++j) store16(&Ost[(srow + RPI * j) * OS + schunk * 8], qst[j]);
       __builtin_amdgcn_wave_barrier();
       if (sub + SEL_WG_ROWS < row_hi) fetch_q(qst, tok_next, sub + SEL_WG_ROWS);
-    } else {
-      const int rc_ = min(r, row_hi - 1);
-      const uint32_t head_ = (uint32_t)(rc_ - div_group(rc_, p.g, p.g_shift) * p.g);
-      // k-step ks contracts dims [16 ks, 16 ks + 16): the two lanes of a row read 32 contiguous bytes and a
-      // cache line is used up by four consecutive loads
-      const T* qrow = qbase_row + ((uint64_t)(uint32_t)token * q_sn32 + (head_ * q_sh32 + hh * 8));
-#pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) qdir[ks] = load16<vec8>(qrow + ks * 16);
     }
     f32x16 acc[NA];
 #pragma unroll
@@ -198,6 +201,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
       }
     }
     __builtin_amdgcn_wave_barrier();  // Q fragments consumed: the tile is reused for the output rows
+    if (!STAGED && sub + SEL_WG_ROWS < row_hi) fetch_dir(tok_next, sub + SEL_WG_ROWS);
     // causal mask: key index inside the block must be <= limit
     const int limit = (token - seq_start) - b_local * BK;
     float mx = -INFINITY;
@@ -277,6 +281,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   if (sub >= row_hi) return;
   int ta = row_token(sub);
   if (STAGED) fetch_q(qst, ta, sub);
+  else fetch_dir(ta, sub);
   int tb = sub + SEL_WG_ROWS < row_hi ? row_token(sub + SEL_WG_ROWS) : 0;
   for (; sub < row_hi; sub += SEL_WG_ROWS) {
     const int tc = sub + 2 * SEL_WG_ROWS < row_hi ? row_token(sub + 2 * SEL_WG_ROWS) : 0;
