@@ -43,6 +43,8 @@ CASES = [
     # head dims without a kernel of their own (zero-padded to the next size up)
     ([0, 800], 4, 2, 96, 64, 8, torch.bfloat16, 1.0),
     ([0, 500], 2, 2, 192, 64, 4, torch.bfloat16, 0.5),
+    # empty sequences at the start, in the middle and at the end of the batch; GQA group of 16
+    ([0, 0, 300, 300, 1100, 1100], 16, 1, 128, 64, 8, torch.bfloat16, 1.0),
 ]
 
 

@@ -62,6 +62,7 @@ CASES = [
     ([0, 800], 4, 2, 96, 64, 8, torch.bfloat16),
     ([0, 600], 2, 1, 40, 32, 4, torch.float16),
     ([0, 500], 2, 2, 192, 64, 4, torch.bfloat16),
+    ([0, 0, 300, 300, 1100, 1100], 16, 1, 128, 64, 8, torch.bfloat16),   # empty sequences, GQA group of 16
 ]
 
 
