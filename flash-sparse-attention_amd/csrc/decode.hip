@@ -45,6 +45,10 @@ struct DecParams {
   const int32_t* pos;       // compressed mode: position of the query
   const int32_t* topk_idx;  // selected mode: [Hkv, B, T]
   int batch, hq, hkv, g, topk, block_size, kernel_size, kernel_stride;
+  // One launch covers the heads [head0, head0 + g) of every GQA group of gq heads (the 16 columns of the MFMA tile
+  // hold at most 16 heads): groups of more heads are served by several launches over the same workspace.
+  int gq, head0;
+  int score_col;            // compressed mode with raw_score: the column whose unscaled scores are kept
   float scale_log2;
   void* o;                  // [B, Hq, D] contiguous
   float* lse;               // [Hq, B]
@@ -181,8 +185,8 @@ decode_attn_kernel(DecParams p) {
   vec8 qreg[NS];
   auto load_q = [&](int b, int h) {
     int hq_i = -1;
-    if (l16 < p.g) hq_i = h * p.g + l16;
-    else if (MODE == DEC_MODE_COMPRESSED && l16 == p.g) hq_i = p.score_head_as_written ? h : h * p.g;
+    if (l16 < p.g) hq_i = h * p.gq + p.head0 + l16;
+    else if (MODE == DEC_MODE_COMPRESSED && p.raw_score && l16 == p.score_col) hq_i = h;  // as written: head h of q
     const T* qrow = reinterpret_cast<const T*>(p.q) + (int64_t)b * p.q_sb + (int64_t)max(hq_i, 0) * p.q_sh + 8 * kg;
 #pragma unroll
     for (int s_ = 0; s_ < NS; ++s_) qreg[s_] = hq_i >= 0 ? load16<vec8>(qrow + 32 * s_) : zero8<T>();
@@ -247,7 +251,7 @@ decode_attn_kernel(DecParams p) {
         }
       }
       __builtin_amdgcn_wave_barrier();
-      if (MODE == DEC_MODE_COMPRESSED && p.raw_score && l16 == p.g) {
+      if (MODE == DEC_MODE_COMPRESSED && p.raw_score && l16 == p.score_col) {
         float* rs = p.raw_score + ((int64_t)h * p.batch + rq.b) * p.raw_ld + row0;
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
@@ -361,7 +365,7 @@ decode_merge_kernel(DecParams p, int D, int n_waves) {
         }
     }
     const float inv_l = lt > 0.f ? 1.f / lt : 0.f;
-    const int hq_i = h * p.g + col;
+    const int hq_i = h * p.gq + p.head0 + col;
     reinterpret_cast<T*>(p.o)[((int64_t)b * p.hq + hq_i) * D + d] = (T)(o * inv_l);
     if (d == 0) p.lse[(int64_t)hq_i * p.batch + b] = lt > 0.f ? mt + log2f(lt) : -INFINITY;
   }
@@ -492,15 +496,28 @@ static int dec_grid_waves(int* n_waves) {
   return 0;
 }
 
+// p0.g holds the whole group size on entry.  Scores of the scoring head: with the first head of the group as
+// scoring head they are the scores of column 0 of the first launch; with the head that the reference's kernel
+// actually reads (q head number h for kv head h) they need a column of their own, so that launch has 15 heads.
 template <typename T, int D, int MODE>
-static int dec_launch(const DecParams& p, hipStream_t stream) {
+static int dec_launch(const DecParams& p0, hipStream_t stream) {
   int n_waves = 0;
   int rc = dec_grid_waves<T, D, MODE>(&n_waves);
   if (rc) return rc;
   ProfScope ps_(MODE == DEC_MODE_COMPRESSED ? "decode_cmpattn" : "decode_selattn", stream);
+  DecParams p = p0;
+  p.gq = p0.g;
   if (MODE == DEC_MODE_COMPRESSED) decode_plan_kernel<MODE><<<1, WAVE, 0, stream>>>(p);
-  decode_attn_kernel<T, D, MODE><<<n_waves, WAVE, DecLds<D>::BYTES, stream>>>(p);
-  decode_merge_kernel<T, MODE><<<dim3(p.batch, p.hkv), 256, 0, stream>>>(p, D, n_waves);
+  for (int head0 = 0; head0 < p0.g;) {
+    p.head0 = head0;
+    p.raw_score = head0 == 0 ? p0.raw_score : nullptr;
+    const bool own_col = MODE == DEC_MODE_COMPRESSED && p.raw_score && p0.score_head_as_written;
+    p.g = std::min(p0.g - head0, own_col ? 15 : 16);
+    p.score_col = own_col ? p.g : 0;
+    decode_attn_kernel<T, D, MODE><<<n_waves, WAVE, DecLds<D>::BYTES, stream>>>(p);
+    decode_merge_kernel<T, MODE><<<dim3(p.batch, p.hkv), 256, 0, stream>>>(p, D, n_waves);
+    head0 += p.g;
+  }
   return 0;
 }
 
@@ -581,7 +598,6 @@ extern "C" int fsa_decode_cmpattn(const void* q, const void* ck, const void* cv,
   FSA_CHECK_ARG(num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
                 "fsa_decode_cmpattn: num_q_heads must be a multiple of num_kv_heads");
   const int g = num_q_heads / num_kv_heads;
-  FSA_CHECK_ARG(g <= 15, "fsa_decode_cmpattn: at most 15 query heads per kv head");
   FSA_CHECK_ARG(max_keys >= 0 && max_keys < (1ll << 30), "fsa_decode_cmpattn: bad max_keys");
   FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim),
                 "fsa_decode_cmpattn: workspace too small (see fsa_decode_workspace_bytes)");
@@ -645,7 +661,6 @@ extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void
   FSA_CHECK_ARG(dtype == FSA_BF16 || dtype == FSA_FP16, "fsa_decode_selattn: dtype must be bf16 or fp16");
   FSA_CHECK_ARG(num_kv_heads >= 1 && num_q_heads % num_kv_heads == 0,
                 "fsa_decode_selattn: num_q_heads must be a multiple of num_kv_heads");
-  FSA_CHECK_ARG(num_q_heads / num_kv_heads <= 16, "fsa_decode_selattn: at most 16 query heads per kv head");
   FSA_CHECK_ARG(batch >= 1 && topk >= 1 && block_size >= 1, "fsa_decode_selattn: bad sizes");
   FSA_CHECK_ARG(workspace && workspace_bytes >= dec_ws_bytes(batch, num_q_heads, num_kv_heads, head_dim),
                 "fsa_decode_selattn: workspace too small (see fsa_decode_workspace_bytes)");

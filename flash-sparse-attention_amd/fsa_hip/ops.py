@@ -281,6 +281,8 @@ def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_
     nblk = (int(max_seqlen_q) + block_size - 1) // block_size
     t_out = min(topk, nblk)
     dev = q.device
+    if ck.shape[0] == 0:   # no compressed key in the whole batch: the lengths in cu_k are zero, this row is never read
+        ck = torch.zeros((1, hkv, d), dtype=q.dtype, device=dev)
     idx = torch.empty((hkv, n, t_out), dtype=torch.int32, device=dev)
     bscore = torch.empty((hkv, n, nblk), dtype=torch.float32, device=dev) if return_block_score else None
     score_cols = max(1, int(max_seqlen_k))

@@ -261,8 +261,10 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
  * fsa_decode_workspace_bytes(...) bytes (max_keys is kept for compatibility
  * and does not change the size).  max_keys of fsa_decode_cmpattn is a host
  * upper bound of the visible compressed cache of one request (keys beyond it
- * are ignored).  At most 15 (compressed) / 16 (selected) query heads per kv
- * head.
+ * are ignored).  One launch serves up to 16 query heads per kv head; larger
+ * GQA groups (and groups of 16 when score_head_as_written asks for a score
+ * column of its own) are served by several launches inside the call, each of
+ * which reads the keys again.
  * ---------------------------------------------------------------------- */
 size_t fsa_decode_workspace_bytes(int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
                                   int32_t head_dim, int64_t max_keys);

@@ -180,3 +180,26 @@ def test_cmp_topk_variants(dev, case):
         seg = idx[:, a:b]
         assert (seg[..., 0] == 0).all()
         assert (seg == own[None, :, None]).any(-1).all()
+
+
+def test_no_compressed_key_in_the_batch(dev):
+    """Every sequence is shorter than one compression window: the compressed attention output is zero with LSE -inf,
+    and the selection consists of the forced blocks alone."""
+    cu, hq, hkv, d, ks, st, bk, t = [0, 17, 48, 79], 4, 2, 64, 32, 16, 16, 4
+    gen = torch.Generator().manual_seed(3)
+    q = torch.randn(cu[-1], hq, d, generator=gen).to(torch.bfloat16).to(dev)
+    ck = torch.zeros(0, hkv, d, dtype=torch.bfloat16, device=dev)
+    cu_q = torch.tensor(cu, dtype=torch.int32, device=dev)
+    cu_k = torch.zeros(len(cu), dtype=torch.int32, device=dev)
+    o, lse = ops.cmpattn_fwd(q, ck, ck, ks, st, cu_q, cu_k, 31)
+    idx, bscore = ops.cmp_topk(q, ck, lse, ks, st, bk, t, cu_q, cu_k, 31, 0, init_blocks=1, local_blocks=2,
+                               return_block_score=True)
+    torch.cuda.synchronize()
+    assert (o == 0).all() and torch.isinf(lse).all() and (lse < 0).all()
+    want = orc.topk_select_ref(bscore.cpu(), t, cu, bk, to_bf16=False)
+    assert torch.equal(idx.cpu(), want)
+    for a, b in zip(cu[:-1], cu[1:]):
+        own = (torch.arange(b - a) // bk).to(torch.int32)
+        seg = idx.cpu()[:, a:b]
+        assert (seg[..., 0] == 0).all() and (seg == own[None, :, None]).any(-1).all()
+        assert ((seg <= own[None, :, None]) | (seg == -1)).all()

@@ -39,6 +39,8 @@ CASES = [
     ([31, 5000], 4, 4, 128, 64, 16, torch.bfloat16),              # first request has no compressed key
     ([3000, 900, 1500], 6, 2, 64, 32, 8, torch.float16),          # g = 3, block 32
     ([2048, 4100], 4, 2, 256, 128, 8, torch.float16),
+    ([1300, 40, 2600], 32, 2, 128, 64, 8, torch.bfloat16),        # GQA group of 16: one launch, or 15 + 1 heads
+    ([900, 3000], 20, 1, 64, 64, 8, torch.float16),               # GQA group of 20: two launches
 ]
 
 
