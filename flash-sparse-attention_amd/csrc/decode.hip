@@ -44,6 +44,7 @@ struct DecParams {
   const int32_t* cu_k;      // [B+1] rows of k / v per request
   const int32_t* pos;       // compressed mode: position of the query
   const int32_t* topk_idx;  // selected mode: [Hkv, B, T]
+  const int32_t* seqlens;   // selected mode, optional: [B] valid rows of each request's slot (null: the whole slot)
   int batch, hq, hkv, g, topk, block_size, kernel_size, kernel_stride;
   // One launch covers the heads [head0, head0 + g) of every GQA group of gq heads (the 16 columns of the MFMA tile
   // hold at most 16 heads): groups of more heads are served by several launches over the same workspace.
@@ -141,6 +142,7 @@ decode_attn_kernel(DecParams p) {
     r.b = b;
     r.k0 = p.cu_k[b];
     r.len = p.cu_k[b + 1] - r.k0;
+    if (MODE == DEC_MODE_SELECTED && p.seqlens) r.len = max(0, min(r.len, p.seqlens[b]));
     r.nt = dec_tiles<MODE>(p, b, r.len, r.n_keys, r.tpb);
   };
   // first cache row and number of valid keys (0: nothing to do) of a tile
@@ -653,8 +655,8 @@ extern "C" int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const flo
 extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
                                   int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n,
                                   int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
-                                  const int32_t* cu_k, const int32_t* topk_idx, int32_t batch,
-                                  int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                  const int32_t* cu_k, const int32_t* seqlens, const int32_t* topk_idx,
+                                  int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                                   int32_t topk, int32_t block_size, float softmax_scale, void* o,
                                   float* lse, void* workspace, size_t workspace_bytes, void* stream_) {
   FSA_CHECK_ARG(q && k_cache && v_cache && cu_k && topk_idx && o && lse, "fsa_decode_selattn: null pointer");
@@ -667,8 +669,8 @@ extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void
   DecParams p = {};
   p.q = q; p.k = k_cache; p.v = v_cache; p.q_sb = q_stride_b; p.q_sh = q_stride_h;
   p.k_sn = k_stride_n; p.k_sh = k_stride_h; p.v_sn = v_stride_n; p.v_sh = v_stride_h;
-  p.cu_k = cu_k; p.topk_idx = topk_idx; p.batch = batch; p.hq = num_q_heads; p.hkv = num_kv_heads;
-  p.g = num_q_heads / num_kv_heads; p.topk = topk; p.block_size = block_size;
+  p.cu_k = cu_k; p.seqlens = seqlens; p.topk_idx = topk_idx; p.batch = batch; p.hq = num_q_heads;
+  p.hkv = num_kv_heads; p.g = num_q_heads / num_kv_heads; p.topk = topk; p.block_size = block_size;
   p.scale_log2 = softmax_scale * LOG2E; p.o = o; p.lse = lse;
   p.tile_prefix = (int32_t*)workspace; p.part = (float*)((char*)workspace + dec_ws_prefix_bytes(batch));
   int rc = dec_dispatch<DEC_MODE_SELECTED>(dtype, head_dim, p, (hipStream_t)stream_);
@@ -680,8 +682,8 @@ extern "C" int fsa_decode_selattn(const void* q, const void* k_cache, const void
 extern "C" int fsa_decode_selattn_static(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
                                          int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n,
                                          int64_t k_stride_h, int64_t v_stride_n, int64_t v_stride_h,
-                                         const int32_t* cu_k, const int32_t* topk_idx, int32_t batch,
-                                         int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                         const int32_t* cu_k, const int32_t* seqlens, const int32_t* topk_idx,
+                                         int32_t batch, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                                          int32_t topk, int32_t block_size, float softmax_scale, void* o,
                                          float* lse, void* stream_) {
   FSA_CHECK_ARG(batch >= 1 && num_kv_heads >= 1 && num_q_heads >= 1 && num_q_heads % num_kv_heads == 0 &&
@@ -700,6 +702,6 @@ extern "C" int fsa_decode_selattn_static(const void* q, const void* k_cache, con
   // every partial slot that the merge reads is written by the attention kernel of the same call: nothing in the
   // buffer has to start at zero
   return fsa_decode_selattn(q, k_cache, v_cache, dtype, q_stride_b, q_stride_h, k_stride_n, k_stride_h, v_stride_n,
-                            v_stride_h, cu_k, topk_idx, batch, num_q_heads, num_kv_heads, head_dim, topk, block_size,
+                            v_stride_h, cu_k, seqlens, topk_idx, batch, num_q_heads, num_kv_heads, head_dim, topk, block_size,
                             softmax_scale, o, lse, scratch, DEC_STATIC_SCRATCH_BYTES, stream_);
 }

@@ -70,9 +70,9 @@ SIGNATURES = {
                                      i32, i32, i32, i32, i32, i32, f32, i32, i64, vp, vp, vp, i64, vp, sz, vp]),
     "fsa_decode_topk": (C.c_int, [vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32,
                                   i32, i32, i32, i32, i32, f32, i64, vp, vp, vp]),
-    "fsa_decode_selattn": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp,
+    "fsa_decode_selattn": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp, vp,
                                      i32, i32, i32, i32, i32, i32, f32, vp, vp, vp, sz, vp]),
-    "fsa_decode_selattn_static": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp,
+    "fsa_decode_selattn_static": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp, vp,
                                             i32, i32, i32, i32, i32, i32, f32, vp, vp, vp]),
 }
 

@@ -357,9 +357,11 @@ def decode_topk(raw_score, lse, cu_ck, pos, seqlens, num_q_heads, kernel_size, k
     return (idx, bscore) if return_block_score else idx
 
 
-def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scale=None):
-    """Decode-step selected attention: (o [B,Hq,D], lse [Hq,B])."""
+def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scale=None, seqlens=None):
+    """Decode-step selected attention: (o [B,Hq,D], lse [Hq,B]).  `seqlens` (optional, int32 [B] on the device):
+    valid rows of each request's slot [cu_k[b], cu_k[b+1]) of the caches; default: the whole slot."""
     _require_cuda(q, k_cache, v_cache, cu_k, topk_idx)
+    assert seqlens is None or (seqlens.is_cuda and seqlens.dtype == torch.int32 and seqlens.numel() == q.shape[0])
     assert q.dtype in _DTYPE and q.dtype == k_cache.dtype == v_cache.dtype
     assert topk_idx.dtype == torch.int32 and topk_idx.is_contiguous()
     assert q.stride(2) == 1 and k_cache.stride(2) == 1 and v_cache.stride(2) == 1
@@ -372,7 +374,7 @@ def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scal
     dn = _native_dim(d)
     if dn != d:
         o, lse = decode_selattn(_pad_d(q, dn), _pad_d(k_cache, dn), _pad_d(v_cache, dn), cu_k, topk_idx, block_size,
-                                softmax_scale)
+                                softmax_scale, seqlens)
         return _cut_d(o, d), lse
     dev = q.device
     o = torch.empty((b, hq, d), dtype=q.dtype, device=dev)
@@ -382,13 +384,13 @@ def decode_selattn(q, k_cache, v_cache, cu_k, topk_idx, block_size, softmax_scal
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     rc = lib.fsa_decode_selattn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _DTYPE[q.dtype], q.stride(0), q.stride(1),
                                 k_cache.stride(0), k_cache.stride(1), v_cache.stride(0), v_cache.stride(1),
-                                _ptr(cu_k), _ptr(topk_idx), b, hq, hkv, d, topk_idx.shape[2], block_size,
+                                _ptr(cu_k), _ptr(seqlens), _ptr(topk_idx), b, hq, hkv, d, topk_idx.shape[2], block_size,
                                 float(softmax_scale), _ptr(o), _ptr(lse), _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_decode_selattn")
     return o, lse
 
 
-def decode_selattn_static(q, k_cache, v_cache, cu_k, topk_idx, block_size, o, lse, softmax_scale=None):
+def decode_selattn_static(q, k_cache, v_cache, cu_k, topk_idx, block_size, o, lse, softmax_scale=None, seqlens=None):
     """Decode-step selected attention into caller-provided `o` [B,Hq,D] and `lse` [Hq,B], with the partial results
     in the library's built-in scratch buffer: the call allocates nothing (C entry point fsa_decode_selattn_static).
     Raises if the sizes exceed the buffer."""
@@ -406,7 +408,7 @@ def decode_selattn_static(q, k_cache, v_cache, cu_k, topk_idx, block_size, o, ls
         softmax_scale = 1.0 / math.sqrt(d)
     rc = lib.fsa_decode_selattn_static(_ptr(q), _ptr(k_cache), _ptr(v_cache), _DTYPE[q.dtype], q.stride(0),
                                        q.stride(1), k_cache.stride(0), k_cache.stride(1), v_cache.stride(0),
-                                       v_cache.stride(1), _ptr(cu_k), _ptr(topk_idx), b, hq, hkv, d,
+                                       v_cache.stride(1), _ptr(cu_k), _ptr(seqlens), _ptr(topk_idx), b, hq, hkv, d,
                                        topk_idx.shape[2], block_size, float(softmax_scale), _ptr(o), _ptr(lse),
                                        _stream(q.device))
     _lib.check(rc, "fsa_decode_selattn_static")

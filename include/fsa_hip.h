@@ -250,7 +250,11 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
  * fsa_decode_selattn replaces _topk_sparse_attention_decode
  * (fsa_preview/ops/selected_attention_decode.py:8-42): the g heads of a group
  * attend every cached key of the selected blocks (ids < 0, past the cache or
- * repeated are ignored).
+ * repeated are ignored).  Request b owns rows [cu_k[b], cu_k[b+1]) of the
+ * caches; seqlens (optional, [B] on the device, may be null) gives the number
+ * of those rows that hold tokens, for callers that keep every request in a
+ * slot of fixed capacity and let it grow (a step recorded into a HIP graph
+ * stays valid while the lengths change in device memory).
  *
  * Both attention calls run a grid of single-wave work-groups that stays
  * resident for the whole launch; the key tiles of all (request, kv head) pairs
@@ -287,7 +291,7 @@ int fsa_decode_topk(const float* raw_score, int64_t raw_ld, const float* lse, co
 
 int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
                        int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
-                       int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_k,
+                       int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_k, const int32_t* seqlens,
                        const int32_t* topk_idx, int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
                        int32_t head_dim, int32_t topk, int32_t block_size, float softmax_scale, void* o,
                        float* lse, void* workspace, size_t workspace_bytes, void* stream);
@@ -307,7 +311,7 @@ int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, 
 int fsa_decode_selattn_static(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
                               int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,
                               int64_t v_stride_n, int64_t v_stride_h, const int32_t* cu_k,
-                              const int32_t* topk_idx, int32_t batch, int32_t num_q_heads,
+                              const int32_t* seqlens, const int32_t* topk_idx, int32_t batch, int32_t num_q_heads,
                               int32_t num_kv_heads, int32_t head_dim, int32_t topk, int32_t block_size,
                               float softmax_scale, void* o, float* lse, void* stream);
 
