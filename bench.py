@@ -275,13 +275,28 @@ def side_workload(args):
         kern[nm] = kern.get(nm, 0.0) + t_
     kernels = _kernel_records(kern, algo)
     lib_ms = sum(kern.values())
+    extra = {}
+    if args.workload == "decode":
+        # the same step recorded into a HIP graph (the lengths are device arrays, so a recorded step stays valid
+        # while the caches grow): what the launches cost when they are issued one by one
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        extra["graph_replay_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / args.steps, 4)
     print(json.dumps({"metric": "ms per step", "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps,
                       "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": False,
                       "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
                       "config": {"workload": name},
                       "library_kernels_ms_total": round(lib_ms, 4),
                       "other_ms": round(ms - lib_ms, 4),   # projections on the BLAS library, autograd glue
-                      "kernels": kernels}))
+                      **extra, "kernels": kernels}))
 
 
 def main():
