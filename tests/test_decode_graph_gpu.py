@@ -76,3 +76,28 @@ def test_decode_step_graph_replays_equal_eager(dev):
         pos += 37                                    # the caches grow between the replays
         seqlens += 37
         q.copy_(torch.randn(nreq, hq, d, generator=gen).to(torch.bfloat16))
+
+
+def test_selected_decode_with_slot_lengths(dev):
+    """`seqlens` cuts every request to its valid rows: equal to the packed caches; a request with no valid row gives
+    a zero output row with LSE -inf; block ids past the valid rows are ignored."""
+    hq, hkv, d, bk, t = 4, 2, 64, 32, 4
+    cap = [300, 200, 500]
+    lens = [257, 0, 31]
+    gen = torch.Generator().manual_seed(4)
+    cu = [0]
+    for c in cap:
+        cu.append(cu[-1] + c)
+    q = torch.randn(3, hq, d, generator=gen).to(torch.float16).to(dev)
+    kc, vc = (torch.randn(cu[-1], hkv, d, generator=gen).to(torch.float16).to(dev) for _ in range(2))
+    idx = torch.tensor([[[0, 8, 3, 9], [0, 1, -1, -1], [0, 1, 2, -1]]] * hkv, dtype=torch.int32, device=dev)  # 9, 1, 2: past the rows
+    cu_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    sl = torch.tensor(lens, dtype=torch.int32, device=dev)
+    o, lse = ops.decode_selattn(q, kc, vc, cu_t, idx, bk, seqlens=sl)
+    rows = torch.cat([torch.arange(cu[b], cu[b] + lens[b]) for b in range(3)]).to(dev)
+    cu_p = torch.tensor([0, 257, 257, 288], dtype=torch.int32, device=dev)
+    o_p, lse_p = ops.decode_selattn(q, kc[rows], vc[rows], cu_p, idx, bk)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o_p) and torch.equal(lse, lse_p)
+    assert (o[1] == 0).all() and torch.isinf(lse[:, 1]).all() and (lse[:, 1] < 0).all()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse[:, [0, 2]]).all()
