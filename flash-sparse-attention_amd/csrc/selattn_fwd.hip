@@ -205,15 +205,20 @@ selattn_fwd_main_kernel(SelFwdParams p) {
     // causal mask: key index inside the block must be <= limit
     const int limit = (token - seq_start) - b_local * BK;
     float mx = -INFINITY;
+    // only the rows of the block's own queries see it partly: a wave without such a row skips the mask
+    if (!__all(limit >= BK - 1)) {
+#pragma unroll
+      for (int a = 0; a < NA; ++a)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+          if (key > limit) acc[a][i] = -INFINITY;
+        }
+    }
 #pragma unroll
     for (int a = 0; a < NA; ++a)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = a * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
-        float sv = key <= limit ? acc[a][i] : -INFINITY;
-        acc[a][i] = sv;
-        mx = fmaxf(mx, sv);
-      }
+      for (int i = 0; i < 16; ++i) mx = fmaxf(mx, acc[a][i]);
     mx = fmaxf(mx, xor32(mx));
     const float mref = (mx == -INFINITY) ? 0.f : mx * p.scale_log2;
     float l = 0.f;
