@@ -236,16 +236,24 @@ selattn_fwd_main_kernel(SelFwdParams p) {
     const int64_t prow = prow0 + r;
     // O^T accumulators -> this wave's LDS tile [row][d] -> 16-byte stores in which 16 lanes
     // cover one full 2*D-byte row (8 cache lines per store instruction instead of 64)
+    // the products of the next 32 dims are issued before the current ones are converted and stored: the matrix
+    // unit works on them while the vector unit, the LDS and the stores deal with the finished accumulator
+    auto pv = [&](int dt) {
+      f32x16 acc_;
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
-      f32x16 oacc;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[i] = 0.f;
+      for (int i = 0; i < 16; ++i) acc_[i] = 0.f;
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
         vec8 vf = lds_read_tr8<T>(vtr + 16 * j * VS + dt * 32, 8 * VS);
-        oacc = Elem<T>::mfma32(vf, pk[j], oacc);
+        acc_ = Elem<T>::mfma32(vf, pk[j], acc_);
       }
+      return acc_;
+    };
+    f32x16 onext = pv(0);
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      const f32x16 oacc = onext;
+      if (dt + 1 < NDT) onext = pv(dt + 1);
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         typename Elem<T>::vec4 x;
