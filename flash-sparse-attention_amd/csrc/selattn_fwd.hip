@@ -269,7 +269,8 @@ selattn_fwd_main_kernel(SelFwdParams p) {
         for (int j = 0; j < 2; ++j) {
           const int row = (lane >> 2) + 16 * j;
           vec8 y = load16<vec8>(&Osl[row * SLS + (lane & 3) * 8]);
-          if (sub + row < row_hi) store16_stream(opart + (prow0 + sub + row) * D + dt * 32 + (lane & 3) * 8, y);
+          // 64-byte pieces: left to the L2 to merge into whole lines (as non-temporal stores they cost 4 % more)
+          if (sub + row < row_hi) store16(opart + (prow0 + sub + row) * D + dt * 32 + (lane & 3) * 8, y);
         }
         __builtin_amdgcn_wave_barrier();
       }
