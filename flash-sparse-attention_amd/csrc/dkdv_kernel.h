@@ -487,14 +487,38 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
     for (int u = 0; u < NU; ++u) {
       vec8 pb = __builtin_shufflevector(pk[2 * u], pk[2 * u + 1], 0, 1, 2, 3, 4, 5, 6, 7);
       vec8 dsb = __builtin_shufflevector(dsk[2 * u], dsk[2 * u + 1], 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-      for (int t = 0; t < NDT; ++t) {
+      // The operands of d tile t + 1 are requested before the products of d tile t are issued, one tile ahead and no
+      // more: left to itself the compiler fetches the whole second half of the rows ahead (64 registers) and then
+      // waits for each operand of the first half right after requesting it.
+      auto rd = [&](int t, int which) {
         const T* trp = lds_ptr<T>(tr_addr0 ^ (32u * t));
-        vec8 doa = lds_read_tr8<T>(trp + (O_BYTES / 2 + 32 * u * QS), 16 * QS);
-        dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
-        vec8 qa = lds_read_tr8<T>(trp + 32 * u * QS, 16 * QS);
-        dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
-        if (C::TIGHT_REGS && (t & 1) == 1) asm volatile("" ::: "memory");  // keep the operand reads from piling up
+        return lds_read_tr8<T>(trp + ((which ? O_BYTES / 2 : 0) + 32 * u * QS), 16 * QS);
+      };
+      if constexpr (D <= 128) {
+        vec8 doa = rd(0, 1), qa = rd(0, 0);
+#pragma unroll
+        for (int t = 0; t < NDT; ++t) {
+          vec8 doa_n = doa, qa_n = qa;
+          if (t + 1 < NDT) {
+            doa_n = rd(t + 1, 1);
+            qa_n = rd(t + 1, 0);
+          }
+          dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
+          dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
+          doa = doa_n;
+          qa = qa_n;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      } else {  // head_dim 256: no register to spare for the operands of the next tile
+#pragma unroll
+        for (int t = 0; t < NDT; ++t) {
+          vec8 doa = rd(t, 1);
+          dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
+          vec8 qa = rd(t, 0);
+          dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
+          if (C::TIGHT_REGS && (t & 1) == 1) asm volatile("" ::: "memory");  // keep the operand reads from piling up
+        }
       }
     }
     if (FUSE_DQ) {
