@@ -534,16 +534,11 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
 #pragma unroll
         for (int u = 0; u < BK / 32; ++u)
           dsb[u] = lds_read_tr8<T>(&dSs[32 * u * C::DSS + str_off + 16 * rt], 16 * C::DSS);
-#pragma unroll
-        for (int tt = 0; tt < NTW; ++tt) {
-          const int t = tg * NTW + tt;
-          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int u = 0; u < BK / 32; ++u) {
-            // the K copy is swizzled like the Q tile (same row pattern)
-            vec8 ka = lds_read_tr8<T>(lds_ptr<T>(tr_addr0 ^ (32u * t)) + (K_BYTES / 2 + 32 * u * C::KS), 16 * C::KS);
-            acc = Elem<T>::mfma16(ka, dsb[u], acc);
-          }
+        // the K copy is swizzled like the Q tile (same row pattern)
+        auto kread = [&](int tt, int u) {
+          return lds_read_tr8<T>(lds_ptr<T>(tr_addr0 ^ (32u * (tg * NTW + tt))) + (K_BYTES / 2 + 32 * u * C::KS), 16 * C::KS);
+        };
+        auto put = [&](int tt, const f32x4& acc) {
           vec4 x;
 #pragma unroll
           for (int i = 0; i < 4; ++i) x[i] = (T)acc[i];
@@ -551,7 +546,49 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
             store8(&dQst[l16 * C::DQS + 16 * tt + 4 * kg], x);
           } else {  // LDS too small for the staging tiles: direct 8-byte stores
             const int r = base + rt * 16 + l16;
-            if (r < row_hi) store8(dqpart + (prow0 + r) * D + 16 * t + 4 * kg, x);
+            if (r < row_hi) store8(dqpart + (prow0 + r) * D + 16 * (tg * NTW + tt) + 4 * kg, x);
+          }
+        };
+        if constexpr (D <= 128 && NTW % 2 == 0) {
+          // two d tiles at a time (two independent accumulator chains), the K^T operands of the next two requested
+          // before the products of the current two are issued
+          constexpr int NKU = BK / 32;
+          vec8 ka[2][NKU];
+#pragma unroll
+          for (int u = 0; u < NKU; ++u) {
+            ka[0][u] = kread(0, u);
+            ka[1][u] = kread(1, u);
+          }
+#pragma unroll
+          for (int tt = 0; tt < NTW; tt += 2) {
+            vec8 kn[2][NKU];
+#pragma unroll
+            for (int u = 0; u < NKU; ++u) {
+              kn[0][u] = tt + 2 < NTW ? kread(tt + 2, u) : ka[0][u];
+              kn[1][u] = tt + 2 < NTW ? kread(tt + 3, u) : ka[1][u];
+            }
+            f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < NKU; ++u) {
+              a0 = Elem<T>::mfma16(ka[0][u], dsb[u], a0);
+              a1 = Elem<T>::mfma16(ka[1][u], dsb[u], a1);
+            }
+            put(tt, a0);
+            put(tt + 1, a1);
+#pragma unroll
+            for (int u = 0; u < NKU; ++u) {
+              ka[0][u] = kn[0][u];
+              ka[1][u] = kn[1][u];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        } else {
+#pragma unroll
+          for (int tt = 0; tt < NTW; ++tt) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < BK / 32; ++u) acc = Elem<T>::mfma16(kread(tt, u), dsb[u], acc);
+            put(tt, acc);
           }
         }
         // [16 rows][DW] piece -> row-coalesced 16-byte stores (CPW lanes per row)
