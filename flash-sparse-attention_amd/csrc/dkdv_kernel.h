@@ -594,12 +594,15 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
         // [16 rows][DW] piece -> row-coalesced 16-byte stores (CPW lanes per row)
         __builtin_amdgcn_wave_barrier();
         constexpr int CPW = C::DW / 8, RPI = 64 / CPW;
+        if constexpr (C::STAGE_DQ) {  // all pieces read from the staging tile first, then stored
+          vec8 xs[16 / RPI];
 #pragma unroll
-        for (int j = 0; C::STAGE_DQ && j < 16 / RPI; ++j) {
-          const int row = lane / CPW + RPI * j;
-          const int r = base + rt * 16 + row;
-          vec8 x = load16<vec8>(&dQst[row * C::DQS + (lane % CPW) * 8]);
-          if (r < row_hi) store16_stream(dqpart + (prow0 + r) * D + tg * C::DW + (lane % CPW) * 8, x);
+          for (int j = 0; j < 16 / RPI; ++j) xs[j] = load16<vec8>(&dQst[(lane / CPW + RPI * j) * C::DQS + (lane % CPW) * 8]);
+#pragma unroll
+          for (int j = 0; j < 16 / RPI; ++j) {
+            const int r = base + rt * 16 + lane / CPW + RPI * j;
+            if (r < row_hi) store16_stream(dqpart + (prow0 + r) * D + tg * C::DW + (lane % CPW) * 8, xs[j]);
+          }
         }
         __builtin_amdgcn_wave_barrier();
       }
