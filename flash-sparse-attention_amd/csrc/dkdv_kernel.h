@@ -476,7 +476,8 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       // dS^T[key][row] for the whole tile: every lane owns 4 consecutive rows of its key
 #pragma unroll
       for (int rt = 0; rt < NRT; ++rt) store8(&dSs[key * C::DSS + rt * 16 + 4 * kg], dsk[rt]);
-      __syncthreads();
+      // (the other waves read it in the dQ products only: the barrier stands behind the dK / dV products, which
+      // use the wave's own P and dS, so that a wave that is ahead does not wait here)
     }
     // The two waves of a SIMD are in different phases most of the time.  From here to the end of the pass the wave
     // issues its matrix products back to back (dK / dV, then dQ): raised priority keeps the other wave's vector work
@@ -522,6 +523,7 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       }
     }
     if (FUSE_DQ) {
+      __syncthreads();  // dS^T of all waves is in LDS
       // dQ^T[d][row] = sum over the block's keys of K^T[d][key] dS^T[key][row]; row tiles are
       // dealt round-robin to the waves, both operands come from transposing LDS reads
       T* dqpart = reinterpret_cast<T*>(p.dq_part);
