@@ -610,11 +610,12 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
       }
     }
     if (FUSE_DQ) __builtin_amdgcn_s_setprio(0);
+    // With the fused dQ every wave has passed the barrier above after its last read of the Q / dO tiles (the dQ
+    // products read the dS^T tile and the K copy only): the rows of the next pass go into LDS without another
+    // barrier in front, and one barrier ends the pass.
+    if (!FUSE_DQ) __syncthreads();
+    if (more) stash();
     __syncthreads();
-    if (more) {
-      stash();
-      __syncthreads();
-    }
   }
 
   // accumulators: dV^T[d = 16*t + 4*kg + i][key]
