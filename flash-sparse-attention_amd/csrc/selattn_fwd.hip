@@ -164,7 +164,7 @@ selattn_fwd_main_kernel(SelFwdParams p) {
     }
   };
   constexpr bool STAGED = SelLds<D, BK>::STAGE_OUT;  // false: LDS cannot hold the wave tiles, direct loads / stores
-  vec8 qst[NLD];
+  vec8 qst[NLD], qst_b[NLD];   // staged mode: the rows of the next two sub-tiles wait here (two buffers in turn)
   // Direct mode: the Q fragments of a lane's row in the MFMA operand layout, straight from global memory.  k-step ks
   // contracts dims [16 ks, 16 ks + 16): the two lanes of a row read 32 contiguous bytes and a cache line is used up
   // by four consecutive loads.  Like qst they are requested one sub-tile ahead: as soon as the S^T products have
@@ -177,16 +177,17 @@ selattn_fwd_main_kernel(SelFwdParams p) {
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) qdir[STAGED ? 0 : ks] = load16<vec8>(qrow + ks * 16);
   };
-  // one sub-tile: rows sub.. of the block; qst holds its Q rows (row-coalesced layout) on entry
-  // and those of the next sub-tile (token ids tok_next) on exit
-  auto step = [&](int token, int sub, int tok_next) {
+  // one sub-tile: rows sub.. of the block (direct mode: tok_next = token ids of the next sub-tile)
+  // staged mode: `qbuf` holds the rows of this sub-tile on entry and, once they are parked in LDS, takes the rows
+  // of the sub-tile after the next (token ids tok_next): the gathers of two sub-tiles are in flight at a time
+  auto step = [&](vec8 (&qbuf)[NLD], int token, int sub, int tok_next) {
     const int r = sub + col;
     const bool valid = r < row_hi;
     if (STAGED) {
 #pragma unroll
-      for (int j = 0; j < NLD; ++j) store16(&Ost[(srow + RPI * j) * OS + schunk * 8], qst[j]);
+      for (int j = 0; j < NLD; ++j) store16(&Ost[(srow + RPI * j) * OS + schunk * 8], qbuf[j]);
       __builtin_amdgcn_wave_barrier();
-      if (sub + SEL_WG_ROWS < row_hi) fetch_q(qst, tok_next, sub + SEL_WG_ROWS);
+      if (sub + 2 * SEL_WG_ROWS < row_hi) fetch_q(qbuf, tok_next, sub + 2 * SEL_WG_ROWS);
     }
     f32x16 acc[NA];
 #pragma unroll
@@ -294,12 +295,27 @@ selattn_fwd_main_kernel(SelFwdParams p) {
   int sub = row_lo + wv * 32;
   if (sub >= row_hi) return;
   int ta = row_token(sub);
-  if (STAGED) fetch_q(qst, ta, sub);
-  else fetch_dir(ta, sub);
+  if (STAGED) {
+    auto tok_at = [&](int s_) { return s_ < row_hi ? row_token(s_) : 0; };
+    int tb = tok_at(sub + SEL_WG_ROWS), tc = tok_at(sub + 2 * SEL_WG_ROWS), td = tok_at(sub + 3 * SEL_WG_ROWS);
+    fetch_q(qst, ta, sub);
+    if (sub + SEL_WG_ROWS < row_hi) fetch_q(qst_b, tb, sub + SEL_WG_ROWS);
+    for (;;) {  // two sub-tiles per round, one from each buffer
+      const int te = tok_at(sub + 4 * SEL_WG_ROWS), tf = tok_at(sub + 5 * SEL_WG_ROWS);
+      step(qst, ta, sub, tc);
+      if (sub + SEL_WG_ROWS >= row_hi) break;
+      step(qst_b, tb, sub + SEL_WG_ROWS, td);
+      sub += 2 * SEL_WG_ROWS;
+      if (sub >= row_hi) break;
+      ta = tc; tb = td; tc = te; td = tf;
+    }
+    return;
+  }
+  fetch_dir(ta, sub);
   int tb = sub + SEL_WG_ROWS < row_hi ? row_token(sub + SEL_WG_ROWS) : 0;
   for (; sub < row_hi; sub += SEL_WG_ROWS) {
     const int tc = sub + 2 * SEL_WG_ROWS < row_hi ? row_token(sub + 2 * SEL_WG_ROWS) : 0;
-    step(ta, sub, tb);
+    step(qst, ta, sub, tb);
     ta = tb;
     tb = tc;
   }
