@@ -584,6 +584,18 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
             }
             __builtin_amdgcn_sched_barrier(0);
           }
+        } else if constexpr (NTW % 2 == 0) {  // head_dim 256: pairs of d tiles, no operands held ahead
+#pragma unroll
+          for (int tt = 0; tt < NTW; tt += 2) {
+            f32x4 a0 = {0.f, 0.f, 0.f, 0.f}, a1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < BK / 32; ++u) {
+              a0 = Elem<T>::mfma16(kread(tt, u), dsb[u], a0);
+              a1 = Elem<T>::mfma16(kread(tt + 1, u), dsb[u], a1);
+            }
+            put(tt, a0);
+            put(tt + 1, a1);
+          }
         } else {
 #pragma unroll
           for (int tt = 0; tt < NTW; ++tt) {
