@@ -511,14 +511,26 @@ attn_bwd_dkdv_kernel(SelBwdParams p) {
           __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_sched_barrier(0);
-      } else {  // head_dim 256: no register to spare for the operands of the next tile
+      } else if constexpr (C::NT >= 256) {
+        // head_dim 256: registers for one operand ahead only (dO^T of tile t, Q^T of tile t, dO^T of t + 1, ...);
+        // without it every product waited for operands requested right before it
+        vec8 cur = rd(0, 1);
+#pragma unroll
+        for (int i = 0; i < 2 * NDT; ++i) {
+          vec8 nxt = cur;
+          if (i + 1 < 2 * NDT) nxt = rd((i + 1) / 2, (i + 1) % 2 == 0 ? 1 : 0);
+          if (i % 2 == 0) dvacc[i / 2] = Elem<T>::mfma16(cur, pb, dvacc[i / 2]);
+          else dkacc[i / 2] = Elem<T>::mfma16(cur, dsb, dkacc[i / 2]);
+          cur = nxt;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
 #pragma unroll
         for (int t = 0; t < NDT; ++t) {
           vec8 doa = rd(t, 1);
           dvacc[t] = Elem<T>::mfma16(doa, pb, dvacc[t]);
           vec8 qa = rd(t, 0);
           dkacc[t] = Elem<T>::mfma16(qa, dsb, dkacc[t]);
-          if (C::TIGHT_REGS && (t & 1) == 1) asm volatile("" ::: "memory");  // keep the operand reads from piling up
         }
       }
     }
