@@ -189,15 +189,16 @@ cmpattn_fwd_kernel(CmpParams p) {
     __syncthreads();
     f32x16 acc[NA];
 #pragma unroll
-    for (int a = 0; a < NA; ++a) {
+    for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[a][i] = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
+    for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+      for (int a = 0; a < NA; ++a) {  // consecutive products on different accumulators
         vec8 kf = load16<vec8>(&Ks[(a * 32 + col) * KS + hh * (D / 2) + ks * 8]);
         acc[a] = Elem<T>::mfma32(kf, qreg[ks], acc[a]);
       }
-    }
     const int limit = jmax - jt, limit_lo = jmin - jt;
     float mx = m;
     // tiles that every row of the wave sees completely need no mask
@@ -242,9 +243,9 @@ cmpattn_fwd_kernel(CmpParams p) {
     lsum += xor32(lsum);
     l += lsum;
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt) {
+    for (int j = 0; j < NJ; ++j) {
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
+      for (int dt = 0; dt < NDT; ++dt) {
         vec8 vf = lds_read_tr8<T>(vtr + 16 * j * VS + dt * 32, 8 * VS);
         oacc[dt] = Elem<T>::mfma32(vf, pk[j], oacc[dt]);
       }
@@ -361,9 +362,9 @@ cmpattn_bwd_dq_kernel(CmpParams p) {
         dsk[a * 2 + (i >> 3)][i & 7] = (T)(pv * (dp[a][i] * p.scale - delta_s));
       }
 #pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
+      for (int dt = 0; dt < NDT; ++dt) {
         vec8 kf = lds_read_tr8<T>(ktr + 16 * j * KS + dt * 32, 8 * KS);
         dacc[dt] = Elem<T>::mfma32(kf, dsk[j], dacc[dt]);
       }
