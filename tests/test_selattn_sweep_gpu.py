@@ -50,6 +50,26 @@ def _scramble(topk, seed):
 def test_drawn_configuration(dev, seed):
     cu, hq, hkv, d, bk, t, dtype = _draw(seed)
     print(f"case seed={seed} cu={cu} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    _check(dev, seed, cu, hq, hkv, d, bk, t, dtype)
+
+
+@pytest.mark.parametrize("nseq,maxlen,hkv,g,d,bk,t,dtype", [
+    (1200, 40, 2, 2, 128, 32, 4, torch.bfloat16),
+    (2500, 5, 1, 16, 128, 32, 1, torch.float16),
+    (300, 300, 2, 3, 256, 128, 2, torch.bfloat16),
+])
+def test_many_short_sequences(dev, nseq, maxlen, hkv, g, d, bk, t, dtype):
+    """Batches of hundreds to thousands of sequences of 0 .. maxlen tokens (empty ones included): every sequence
+    is shorter than a few blocks, so most blocks are partial and most selections are forced ones."""
+    rng = np.random.default_rng(nseq)
+    lens = rng.integers(0, maxlen + 1, size=nseq)
+    lens[0] = max(int(lens[0]), 1)
+    cu = [0] + np.cumsum(lens).tolist()
+    print(f"case nseq={nseq} n={cu[-1]} hq={hkv * g} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    _check(dev, nseq, cu, hkv * g, hkv, d, bk, t, dtype, both_index_paths=True)
+
+
+def _check(dev, seed, cu, hq, hkv, d, bk, t, dtype, both_index_paths=False):
     n = cu[-1]
     std = 1.0 if dtype == torch.bfloat16 else 0.5
     q, k, v, do = make_qkv(n, hq, hkv, d, dtype, seed=100 + seed, std=std)
@@ -62,6 +82,15 @@ def test_drawn_configuration(dev, seed):
     assert np.array_equal(index.starts.cpu().numpy()[:, : nb + 1], starts)
     assert np.array_equal(index.sel_tokens.cpu().numpy(), sel_tokens)
     assert np.array_equal(index.slot_of.cpu().numpy(), slot_of)
+    if both_index_paths:
+        import os
+        os.environ["FSA_INDEX_RADIX"] = "1"      # the general (radix sort) path must build the same lists
+        try:
+            other = ops.build_index(topk.to(dev), cu_t.to(dev), bk)
+        finally:
+            os.environ.pop("FSA_INDEX_RADIX")
+        assert torch.equal(other.sel_tokens, index.sel_tokens) and torch.equal(other.slot_of, index.slot_of)
+        assert torch.equal(other.starts, index.starts) and torch.equal(other.counts, index.counts)
 
     qd, kd, vd, dod = (x.to(dev) for x in (q, k, v, do))
     o, lse = ops.selattn_fwd(qd, kd, vd, index)
