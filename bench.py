@@ -40,14 +40,40 @@ TRAFFIC_KERNEL_NAMES = {"selattn_bwd_dqdkdv": "attn_bwd_dkdv_kernel", "selattn_f
                         "selattn_bwd_delta": "selattn_bwd_delta_kernel"}
 
 
+def csrc_sha16() -> str:
+    """Hash of the kernel sources (csrc/*.hip, csrc/*.h, the C header): identifies the code a counter summary
+    was captured from."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "flash-sparse-attention_amd", "csrc")
+    files = sorted(os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
+    files.append(os.path.join(ROOT, "include", "fsa_hip.h"))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        h.update(open(f, "rb").read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(workload: str):
-    """{(label, gqa): bytes per launch} from profiles/<summary>: lines `<kernel> grid=<n> gqa=<g> ... bytes=<x> GB`."""
+    """({(label, gqa): bytes per launch}, source) from profiles/<summary>: lines `<kernel> grid=<n> gqa=<g> ...
+    bytes=<x> GB`.  The summary names the kernel sources it was captured from (`# csrc_sha16: <hash>`); when the
+    sources of this tree differ, nothing is returned - a stale figure is worse than none."""
     import re
     out = {}
-    path = os.path.join(ROOT, "profiles", TRAFFIC_FILES.get(workload, "-"))
+    name = TRAFFIC_FILES.get(workload, "-")
+    path = os.path.join(ROOT, "profiles", name)
     if not os.path.exists(path):
-        return out
-    for line in open(path):
+        return out, None
+    text = open(path).read()
+    m = re.search(r"^# csrc_sha16: (\w+)", text, re.M)
+    sha, now = (m.group(1) if m else None), csrc_sha16()
+    source = {"file": "profiles/" + name, "captured_from_csrc_sha16": sha, "this_tree_csrc_sha16": now,
+              "how": "two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE) over this script, read from the committed "
+                     "summary - not measured in this run"}
+    if sha != now:
+        source["stale"] = True
+        return out, source
+    for line in text.splitlines():
         m = re.match(r"^(\S+)\s+grid=\s*\d+\s+gqa=(\d+)\s.*bytes=([0-9.]+) GB", line)
         if not m:
             continue
@@ -123,6 +149,39 @@ def cpu_baseline(d: int, bk: int, topk: int, hkv: int, c1_seq_len: int, c1_p_key
         "sample_ms": round(t1 * 1e3, 1),
         "gqa1_fwd_bwd_ms": round(t1 * factor * 1e3, 0),
     }
+    return out
+
+
+def parity_sample(run_g, data, g, idx_cpu, bk, n, dtype):
+    """Plain max-abs differences of the device results of one GQA group of the timed workload against the CPU
+    oracle: O / LSE / dQ on 32 seeded queries, dK / dV on key block 0 of kv head 0 (selected by every query: the
+    block with the largest gradients) and on one block in the middle of the sequence.  Part of the CPU-baseline
+    leg: the oracle is the checker here, nothing of it is timed as the product."""
+    import torch
+    from oracle import selattn as orc
+    q, k, v, do = (x.cpu() for x in data[g])
+    dq, dk, dv, o, lse = run_g(g, want_fwd=True)
+    torch.cuda.synchronize()
+    oc, lc = o.float().cpu(), lse.cpu()
+    gen = torch.Generator().manual_seed(7)
+    rows = sorted(set([0, bk, n - 1] + torch.randint(0, n, (29,), generator=gen).tolist()))
+    cu = [0, n]
+    r = orc.selected_attention_rows_ref(q, k, v, idx_cpu, bk, cu, rows, do=do, o_in=oc, lse_in=lc, round_dtype=dtype)
+    out = {"gqa": g, "queries": len(rows),
+           "max_abs_o": float((oc[rows].double() - r["o"]).abs().max()),
+           "max_abs_lse": float((lc[:, rows].double() - r["lse"]).abs().max()),
+           "max_abs_dq": float((dq.float().cpu()[rows].double() - r["dq"]).abs().max())}
+    nblk = (n + bk - 1) // bk
+    for blk in (0, nblk // 2):
+        users = (idx_cpu[0] == blk).any(-1).nonzero().flatten()
+        dk0, dv0 = orc.key_block_grads_ref(q, k, v, do, oc, lc, 0, blk * bk, users, bk, n, round_dtype=dtype)
+        gk = dk[blk * bk:(blk + 1) * bk, 0].float().cpu().double()
+        gv = dv[blk * bk:(blk + 1) * bk, 0].float().cpu().double()
+        out[f"block{blk}"] = {"queries": int(users.numel()), "max_abs_dk": float((gk - dk0).abs().max()),
+                              "max_abs_dv": float((gv - dv0).abs().max()),
+                              "max_ref_dk": float(dk0.abs().max()), "max_ref_dv": float(dv0.abs().max())}
+    out["note"] = ("plain max-abs, no ulp allowance; one bf16 ulp at |ref| = 8 is 0.0625, so the rounding of the "
+                   "output alone can reach 0.031 there")
     return out
 
 
@@ -347,10 +406,11 @@ def main():
     for g in groups:
         data[g] = tuple(x.to(dev) for x in make_qkv(n, hkv * g, hkv, d, dtype, seed=100 + g, std=std))
 
-    def run_g(g):
+    def run_g(g, want_fwd=False):
         q, k, v, do = data[g]
         o, lse, perm = _topk_sparse_attention_fwd_opt(q, k, v, idx, bk, cu_t, cu_t, n, n, scale)
-        return _topk_sparse_attention_bwd_opt(o, do, lse, q, k, v, idx, bk, cu_t, cu_t, n, n, scale, perm)
+        grads = _topk_sparse_attention_bwd_opt(o, do, lse, q, k, v, idx, bk, cu_t, cu_t, n, n, scale, perm)
+        return (*grads, o, lse) if want_fwd else grads
 
     def step():
         for g in groups:
@@ -364,6 +424,19 @@ def main():
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # peak device memory of one group's index + forward + backward (inputs, outputs, index, partial buffers), as
+    # the reference's harness prints it (test/test_FSA_module.py:137)
+    peak_mem = {}
+    for g in groups:
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        r_ = run_g(g)
+        torch.cuda.synchronize()
+        peak_mem[g] = {"max_memory_allocated": int(torch.cuda.max_memory_allocated()),
+                       "above_resident_inputs": int(torch.cuda.max_memory_allocated() - base)}
+        del r_
 
     flops_g = {g: 14.0 * d * p_key * g for g in groups}
     total_tflop = sum(flops_g.values()) / 1e12
@@ -418,7 +491,8 @@ def main():
             return 0.0, by, by
         return 0.0, 0.0, 0.0
 
-    traffic_of = measured_traffic(args.workload) if (n, d, bk, topk) == (65536, 128, 64, 16) else {}
+    traffic_of, traffic_source = (measured_traffic(args.workload) if (n, d, bk, topk) == (65536, 128, 64, 16)
+                                  else ({}, None))
     kernels = []
     for (name, g), ms in sorted(kern.items(), key=lambda kv: -kv[1]):
         fl, by, by_gather = algo(name, g)
@@ -439,7 +513,7 @@ def main():
     dom = kernels[0]
     roofline = {"kernel": f"{dom['kernel']} (GQA {dom['gqa']})", "bound": dom["bound"],
                 "achieved": dom["achieved"], "peak": dom["peak"], "unit": dom["unit"], "frac": dom["frac"],
-                "traffic": dom.get("traffic")}
+                "traffic": dom.get("traffic"), "traffic_source": traffic_source}
     if "hbm" in dom:
         roofline["hbm"] = dom["hbm"]
 
@@ -452,7 +526,13 @@ def main():
         per_gqa.append({"gqa": g, "hq": hkv * g, "index_ms": round(parts.get("index_build", 0), 4),
                         "fwd_ms": round(fwd, 4), "bwd_ms": round(bwd, 4),
                         "tflops": round(flops_g[g] / 1e12 / (tot * 1e-3), 2),
-                        "mfma_frac": round(flops_g[g] / 1e12 / (tot * 1e-3) / MFMA_PEAK_TFLOPS, 4)})
+                        "mfma_frac": round(flops_g[g] / 1e12 / (tot * 1e-3) / MFMA_PEAK_TFLOPS, 4),
+                        **peak_mem[g]})
+    # the binding roofline of the whole step: bytes through the fabric.  least = sum of the kernels' least bytes,
+    # measured = sum of the counter figures (when the committed summary matches this tree)
+    least_total = sum(r.get("hbm", {}).get("least_bytes", r.get("algo_bytes", 0)) for r in kernels)
+    meas = [r.get("traffic") for r in kernels if "algo_bytes" in r]
+    meas_total = sum(meas) if meas and all(meas) else None
 
     out = {
         "metric": METRIC,
@@ -472,12 +552,21 @@ def main():
                    "pairs_per_kv_head": pairs // hkv, "unmasked_qk_pairs_per_q_head": p_key // hkv,
                    "tflop_per_step": round(total_tflop, 4), "seed": 1},
         "mfma_frac_whole_step": round(value / MFMA_PEAK_TFLOPS, 4),
+        "least_bytes_whole_step": int(least_total),
+        "measured_bytes_whole_step": meas_total,
+        "hbm_frac_whole_step": (round(meas_total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
+                                if meas_total else None),
+        "hbm_frac_whole_step_least_bytes": round(least_total / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+        # what the step could reach if every kernel moved only its least bytes at the full HBM peak: the ceiling of a
+        # design that keeps one partial row per (query, block, head) in HBM
+        "design_ceiling_mfma_frac": round(total_tflop / (least_total / (HBM_PEAK_GBS * 1e9)) / MFMA_PEAK_TFLOPS, 4),
         "roofline": roofline,
         "per_gqa": per_gqa,
         "kernels": kernels,
     }
     if not args.no_cpu_baseline and args.workload == "c1":
         out["cpu_baseline"] = cpu_baseline(d, bk, topk, hkv, n, p_key // hkv, args.cpu_seq_len)
+        out["parity_sample"] = parity_sample(run_g, data, max(groups), idx_cpu, bk, n, dtype)
         # the same shape on the GPU, for the speed-up at equal work
         s0 = 4096
         q0, k0, v0 = (x.to(dev) for x in make_qkv(s0, hkv, hkv, d, dtype, seed=0, with_do=False))

@@ -100,7 +100,8 @@ def fsa_layer_ref(params: dict, x, cu_seqlens, cfg: dict, topk_idx=None, table_d
     """fp32 composition of the layer (fsa/module/fsa.py:71-173).  `params` holds the reference's
     parameter names; `cfg` the constructor arguments plus "inv_freq".  When `topk_idx` is given it
     replaces the selection computed from the compressed branch (the selection is discrete, so a
-    like-for-like comparison passes the ids the device chose).  Returns (y, topk_idx, parts)."""
+    like-for-like comparison passes the ids the device chose).  Returns (y, topk_idx, parts);
+    parts["block_score"] holds the fp32 block scores [Hkv, N, nblk] when the selection was computed here."""
     hq, hkv, d = cfg["num_q_heads"], cfg["num_kv_heads"], cfg["head_dim"]
     ks, st, bk, t = cfg["kernel_size"], cfg["kernel_stride"], cfg["block_size"], cfg["topk"]
     xf = x.float()
@@ -128,15 +129,16 @@ def fsa_layer_ref(params: dict, x, cu_seqlens, cfg: dict, topk_idx=None, table_d
     q = rope(q, cu_seqlens)
     ck = rope(ck, cu_k, 0, st)
     o_cmp, lse_cmp = _cmp.compressed_attention_ref(q, ck, cv, ks, st, cu_seqlens, cu_k)
+    block_score = None
     if topk_idx is None:
         max_q = max(b - a for a, b in _bounds(cu_seqlens))
-        topk_idx, _ = _cmp.compressed_topk_ref(q.detach(), ck.detach(), lse_cmp.detach(), ks, st, bk, t, cu_seqlens,
-                                               cu_k, init_blocks=cfg["init_blocks"],
-                                               local_blocks=cfg["local_blocks"], max_seqlen_q=max_q)
+        topk_idx, block_score = _cmp.compressed_topk_ref(q.detach(), ck.detach(), lse_cmp.detach(), ks, st, bk, t,
+                                                         cu_seqlens, cu_k, init_blocks=cfg["init_blocks"],
+                                                         local_blocks=cfg["local_blocks"], max_seqlen_q=max_q)
     k = rope(k, cu_seqlens)
     o_sel, _ = _sel.selected_attention_ref(q, k, v, topk_idx, bk, cu_seqlens)
     o_win, _ = window_attention_ref(q, k, v, cu_seqlens, cfg["window_size"])
     gate = torch.sigmoid(xf @ params["gate.0.weight"].float().t())
     o = gate[:, 0:1, None] * o_cmp + gate[:, 1:2, None] * o_sel + gate[:, 2:3, None] * o_win
     y = o.reshape(o.shape[0], -1) @ params["proj_o.weight"].float().t()
-    return y, topk_idx, {"cmp": o_cmp, "sel": o_sel, "win": o_win, "gate": gate}
+    return y, topk_idx, {"cmp": o_cmp, "sel": o_sel, "win": o_win, "gate": gate, "block_score": block_score}

@@ -7,7 +7,8 @@ fp16; LSE 1e-3).
 
 The gradients are compared with the UNROUNDED oracle that recomputes its own forward (no kernel output enters the
 reference, no rounding point of the kernels is applied): element-wise |got - ref| <= tol + 2 ulp |ref| and a
-relative Frobenius error.  The same independent check runs at two more shapes (GQA 4 ragged batch, fp16 D=256).
+relative Frobenius error.  The same independent check runs at two more shapes (GQA 4 ragged batch, fp16 D=256) and
+on the whole tensors of the headline shape at GQA 1 (S=65536).
 """
 import pytest
 import torch
@@ -28,6 +29,8 @@ CASES = [
     ("C0-fp16", [0, 4096], 4, 4, 128, 64, 16, torch.float16, 1.0),
     ("gqa4-ragged", [0, 1100, 1101, 3000], 8, 2, 128, 64, 16, torch.bfloat16, 1.0),
     ("fp16-d256", [0, 2048], 4, 2, 256, 128, 8, torch.float16, 0.5),
+    # the headline shape at GQA 1, every element of O, LSE, dQ, dK, dV (about a minute of oracle time on the host)
+    ("C1-gqa1-whole", [0, 65536], 4, 4, 128, 64, 16, torch.bfloat16, 1.0),
 ]
 
 
@@ -43,6 +46,8 @@ def test_whole_tensor_against_unrounded_oracle(dev, name, cu, hq, hkv, d, bk, t,
     o, lse = ops.selattn_fwd(qd, kd, vd, index)
     dq, dk, dv = ops.selattn_bwd(qd, kd, vd, o, dod, lse, index)
     torch.cuda.synchronize()
+    print("  device done, oracle running", flush=True)
+    torch.set_num_threads(max(torch.get_num_threads(), min(16, __import__("os").cpu_count() or 1)))
     o_r, lse_r, dq_r, dk_r, dv_r = orc.selected_attention_grads_ref(q.float(), k.float(), v.float(), topk, bk, cu,
                                                                    do.float())
     eo = (o.float().cpu() - o_r).abs().max().item()

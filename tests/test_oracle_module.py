@@ -90,3 +90,27 @@ def test_rope_invariants():
     # the conjugate rotation undoes the rotation
     back = orc.rope_ref(y.double(), cu, inv, conj=True)
     assert torch.allclose(back, x.float(), atol=1e-5)
+
+
+def test_rope_direction_against_complex_multiplication():
+    """The invariants above hold for either rotation sense.  This fixes the sense: the pair
+    (x[d], x[d + D/2]) read as the complex number x[d] + i x[d + D/2] is multiplied by
+    exp(+i * position * inv_freq[d]) (non-interleaved rotary: nsa_ref/module/rope.py:126-134 hands
+    cos/sin of position * inv_freq to a rotate-half rotary).  The opposite sense fails here."""
+    gen = torch.Generator().manual_seed(2)
+    inv = orc.llama3_inv_freq(32, 10000.0, original_max=64)
+    cu = [0, 33, 70]
+    x = torch.randn(70, 3, 32, generator=gen, dtype=torch.float64)
+    for start, stride in ((0, 1), (5, 3)):
+        y = orc.rope_ref(x, cu, inv, start=start, stride=stride)
+        pos = torch.cat([start + torch.arange(33) * stride, start + torch.arange(37) * stride]).double()
+        rot = torch.polar(torch.ones(70, 16, dtype=torch.float64), pos[:, None] * inv.double()[None, :])
+        z = torch.complex(x[..., :16], x[..., 16:]) * rot[:, None, :]
+        assert torch.allclose(y[..., :16].double(), z.real, atol=1e-5)
+        assert torch.allclose(y[..., 16:].double(), z.imag, atol=1e-5)
+        # and the opposite sense is told apart by a margin far above that tolerance
+        zc = torch.complex(x[..., :16], x[..., 16:]) * rot.conj()[:, None, :]
+        assert (y[..., 16:].double() - zc.imag).abs().max() > 0.1
+        # conj=True is exactly that opposite sense
+        yc = orc.rope_ref(x, cu, inv, start=start, stride=stride, conj=True)
+        assert torch.allclose(yc[..., 16:].double(), zc.imag, atol=1e-5)
