@@ -41,6 +41,7 @@ struct CmpParams {
   // score / top-k
   float* score;        // [Hkv, N, score_ld]
   int64_t score_ld;
+  int score_head_step;  // q head that scores kv head h = h * score_head_step (g: first head of the group)
   int rebin;           // cmp_score writes block scores (taps 1 2 2 2 1 over groups of 4 keys) instead of probabilities
 };
 
@@ -483,7 +484,7 @@ cmp_score_kernel(CmpParams p) {
   const int r = row_lo + wv * 32 + col;
   const bool valid = r < lq;
   const int qi = valid ? r : lq - 1;
-  const int hq_i = h * p.g;  // first head of the group
+  const int hq_i = h * p.score_head_step;  // first head of the group (as written: q head = kv head)
   const T* qrow = reinterpret_cast<const T*>(p.q) + (int64_t)(q0 + qi) * p.q_sn + (int64_t)hq_i * p.q_sh + hh * (D / 2);
   vec8 qreg[NKS];
 #pragma unroll
@@ -984,7 +985,8 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
                             int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                             int32_t kernel_size, int32_t kernel_stride, int32_t block_size, int32_t topk,
                             int32_t init_blocks, int32_t local_blocks, int32_t scores_to_bf16,
-                            float softmax_scale, int32_t* topk_idx, float* block_score, void* workspace,
+                            int32_t score_head_as_written, float softmax_scale, int32_t* topk_idx,
+                            float* block_score, void* workspace,
                             size_t workspace_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
   FSA_CHECK_ARG(q && ck && lse && topk_idx && cu_seqlens_q && cu_seqlens_k, "fsa_cmp_topk: null pointer");
@@ -1017,6 +1019,7 @@ extern "C" int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int
   p.g = num_q_heads / num_kv_heads; p.kernel_size = kernel_size; p.kernel_stride = kernel_stride;
   p.scale = softmax_scale; p.scale_log2 = softmax_scale * LOG2E;
   p.rebin = rebin;
+  p.score_head_step = score_head_as_written ? 1 : p.g;
   p.score = (float*)workspace;
   p.score_ld = (score_cols + 3) / 4 * 4;
   rc = cmp_score_dispatch(dtype, head_dim, p, batch, num_kv_heads, max_seqlen_q, stream);

@@ -19,6 +19,8 @@ i32, i64, f32, vp, sz = C.c_int32, C.c_int64, C.c_float, C.c_void_p, C.c_size_t
 SIGNATURES = {
     "fsa_version": (C.c_int, []),
     "fsa_last_error": (C.c_char_p, []),
+    "fsa_native_head_dim": (C.c_int, [i32]),
+    "fsa_pad_head_dim": (C.c_int, [vp, i64, i64, i32, vp, i64, i64, i32, i64, i32, vp]),
     "fsa_profile_enable": (C.c_int, [C.c_int]),
     "fsa_profile_count": (C.c_int, []),
     "fsa_profile_get": (C.c_int, [C.c_int, C.c_char_p, C.c_int, C.POINTER(C.c_float)]),
@@ -49,7 +51,7 @@ SIGNATURES = {
                                   vp, vp, vp, vp, sz, vp]),
     "fsa_cmp_topk_workspace_bytes": (sz, [i64, i32, i64]),
     "fsa_cmp_topk": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, vp, vp, i32,
-                               i64, i64, i64, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, f32,
+                               i64, i64, i64, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, f32,
                                vp, vp, vp, sz, vp]),
     "fsa_winattn_fwd": (C.c_int, [vp, vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, i32, i64, i64,
                                   i32, i32, i32, i32, f32, vp, i64, i64, vp, vp]),

@@ -38,14 +38,30 @@ def _native_dim(d: int, native=_NATIVE_D) -> int:
     raise ValueError(f"head_dim {d} is not supported (at most {native[-1]})")
 
 
+def _resize_d(t: torch.Tensor, d_to: int) -> torch.Tensor:
+    """[..., H, d] -> contiguous [..., H, d_to]: the leading columns copied, the rest zero (fsa_pad_head_dim)."""
+    d = t.shape[-1]
+    rows = t.reshape(-1, t.shape[-2], d) if t.dim() != 3 else t
+    if (t.dtype not in _DTYPE or not t.is_cuda or rows.stride(2) != 1 or d % 4 or d_to % 4
+            or rows.stride(0) % 4 or rows.stride(1) % 4 or t.data_ptr() % 8):
+        # shapes the C helper does not take (fp32 gradients of parameters, odd head dims): torch does the copy
+        return (torch.nn.functional.pad(t, (0, d_to - d)) if d_to > d else t[..., :d_to]).contiguous()
+    out = torch.empty((*t.shape[:-1], d_to), dtype=t.dtype, device=t.device)
+    o3 = out.view(-1, t.shape[-2], d_to)
+    rc = _lib.load().fsa_pad_head_dim(_ptr(rows), rows.stride(0), rows.stride(1), d, _ptr(o3), o3.stride(0),
+                                      o3.stride(1), d_to, rows.shape[0], rows.shape[1], _stream(t.device))
+    _lib.check(rc, "fsa_pad_head_dim")
+    return out
+
+
 def _pad_d(t: Optional[torch.Tensor], d_to: int):
     if t is None or t.shape[-1] == d_to:
         return t
-    return torch.nn.functional.pad(t, (0, d_to - t.shape[-1]))
+    return _resize_d(t, d_to)
 
 
 def _cut_d(t: torch.Tensor, d: int):
-    return t[..., :d].contiguous()
+    return _resize_d(t, d) if t.shape[-1] != d else t
 
 
 def _require_cuda(*tensors):
@@ -265,8 +281,10 @@ def cmpattn_bwd(q, ck, cv, o, do, lse, kernel_size, kernel_stride, cu_q, cu_k, m
 
 def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_k, max_seqlen_q,
              max_seqlen_k, init_blocks=1, local_blocks=2, softmax_scale=None, scores_to_bf16=True,
-             return_block_score=False):
-    """Top-k block ids [Hkv, N, min(topk, nblk)] int32 from the compressed-attention probabilities."""
+             return_block_score=False, score_head_as_written=False):
+    """Top-k block ids [Hkv, N, min(topk, nblk)] int32 from the compressed-attention probabilities of the first
+    q head of every group (score_head_as_written: of q head kh for kv head kh, the literal behaviour of the
+    reference's parallel path, nsa_ref/ops/compressed_attention.py:870, 898, 906)."""
     _require_cuda(q, ck, lse, cu_q, cu_k)
     lib = _lib.load()
     n, hq, d = q.shape
@@ -277,7 +295,7 @@ def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_
     if dn != d:
         return cmp_topk(_pad_d(q, dn), _pad_d(ck, dn), lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_k,
                         max_seqlen_q, max_seqlen_k, init_blocks, local_blocks, softmax_scale, scores_to_bf16,
-                        return_block_score)
+                        return_block_score, score_head_as_written)
     nblk = (int(max_seqlen_q) + block_size - 1) // block_size
     t_out = min(topk, nblk)
     dev = q.device
@@ -295,6 +313,7 @@ def cmp_topk(q, ck, lse, kernel_size, kernel_stride, block_size, topk, cu_q, cu_
                           ck.stride(0), ck.stride(1), _ptr(cu_q), _ptr(cu_k), cu_q.numel() - 1, n,
                           int(max_seqlen_q), max(1, int(max_seqlen_k)), hq, hkv, d, kernel_size, kernel_stride,
                           block_size, topk, init_blocks, local_blocks, 1 if scores_to_bf16 else 0,
+                          1 if score_head_as_written else 0,
                           float(softmax_scale), _ptr(idx), _ptr(bscore), _ptr(ws), ws_bytes, _stream(dev))
     _lib.check(rc, "fsa_cmp_topk")
     return (idx, bscore) if return_block_score else idx

@@ -53,12 +53,18 @@ def compressed_attention(
     init_blocks: int = 1,
     local_blocks: int = 2,
     parallel_topk_compute: Union[str, bool] = False,
+    score_head_as_written: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Attention between the queries and the compressed keys / values, and the top-k block ids
     [num_kv_heads, total_q, min(topk, ceil(max_seqlen_q / block_size))] used by the selected attention.
 
-    `parallel_topk_compute` only decides whether the block scores are rounded to bf16 before the
-    selection (False, the reference's per-head path) or kept in fp32 (True)."""
+    `parallel_topk_compute` decides whether the block scores are rounded to bf16 before the selection
+    (False, the reference's per-head path, the only one its callers use) or kept in fp32 (True).  The
+    reference's parallel path also hands the unsliced q to its score kernel, which then scores kv head
+    kh with q head kh instead of the first head of group kh (nsa_ref/ops/compressed_attention.py:870,
+    898, 906 against :1280-1283); `score_head_as_written=True` together with
+    `parallel_topk_compute=True` reproduces that literally, the default scores every kv head with the
+    first q head of its group on both paths."""
     if max_seqlen_q is None:
         max_seqlen_q = (cu_seqlens_q[1:] - cu_seqlens_q[:-1]).max().item()
     if max_seqlen_k is None:
@@ -76,5 +82,6 @@ def compressed_attention(
     with torch.no_grad():
         topk_idx = _ops.cmp_topk(q, k, lse, kernel_size, kernel_stride, block_size, topk, cu_seqlens_q, cu_seqlens_k,
                                  max_seqlen_q, max_seqlen_k, init_blocks, local_blocks, sm_scale,
-                                 scores_to_bf16=not parallel_topk_compute)
+                                 scores_to_bf16=not parallel_topk_compute,
+                                 score_head_as_written=bool(score_head_as_written and parallel_topk_compute))
     return attn_output, topk_idx

@@ -38,10 +38,30 @@ extern "C" {
 #define FSA_ERR_UNSUPPORTED (-2)
 #define FSA_ERR_WORKSPACE (-3)
 
-/* Library version (major*10000 + minor*100 + patch). */
+/* Library version (major*10000 + minor*100 + patch).  A caller built against an
+ * older header must check it at load: argument lists changed at
+ *   200: fsa_decode_topk (scores_to_bf16 added), fsa_decode_selattn (seqlens added);
+ *   210: fsa_cmp_topk (score_head_as_written added); fsa_native_head_dim and
+ *        fsa_pad_head_dim are new. */
+#define FSA_HIP_VERSION 210
 int fsa_version(void);
 /* Human-readable description of the last error on the calling thread. */
 const char* fsa_last_error(void);
+
+/* Head dims other than 64 / 128 / 256.  The kernels are built for those three;
+ * the reference pads any head_dim <= 256 to the next power of two inside its
+ * kernels (fsa/ops/FSA_topk_sparse_attention.py:692, 760, 904, 1456).  Here the
+ * caller runs the kernels on zero-padded copies: q.k and P.V are unchanged by
+ * zero columns, the softmax scale must be passed explicitly (1/sqrt of the TRUE
+ * head_dim), and the padded columns of outputs and gradients are cut off again.
+ *   fsa_native_head_dim(d): the built size to pad to (d itself if built), -1 if d > 256;
+ *   fsa_pad_head_dim: dst[r, h, 0..d_dst) = src[r, h, 0..min(d_src, d_dst)) then
+ *   zeros, for 16-bit elements - pads (d_dst > d_src) and cuts (d_dst < d_src);
+ *   strides in elements, multiples of 4, d_dst a multiple of 4. */
+int fsa_native_head_dim(int32_t head_dim);
+int fsa_pad_head_dim(const void* src, int64_t src_stride_n, int64_t src_stride_h, int32_t d_src,
+                     void* dst, int64_t dst_stride_n, int64_t dst_stride_h, int32_t d_dst,
+                     int64_t rows, int32_t heads, void* stream);
 
 /* Per-kernel timing for benchmarks (replaces the CUDA-event timer of
  * utils.py:6-27).  While enabled, every kernel launch of the library is
@@ -199,7 +219,10 @@ int fsa_cmpattn_bwd(const void* q, const void* ck, const void* cv, const void* o
  * Replaces _get_attention_score / score_kernel, transform_score /
  * _transform_score_kernel and the torch.topk + sort + mask of
  * nsa_ref/ops/compressed_attention.py:832-1003, 1006-1158, 1272-1315
- * (per kv head, probabilities of the FIRST q head of the group).
+ * (per kv head, probabilities of the FIRST q head of the group; with
+ * score_head_as_written != 0 kv head kh is scored with q head kh instead, which
+ * is what the reference's parallel_topk_compute=True path does when it hands
+ * the unsliced q to score_kernel, compressed_attention.py:870, 898, 906).
  *   topk_idx    [Hkv, total_q, min(topk, nblk)] int32 out, nblk = ceil(max_seqlen_q / block_size)
  *   block_score [Hkv, total_q, nblk] fp32 out, optional (NULL to skip)
  * scores_to_bf16 != 0 rounds the block scores to bf16 before the selection, as
@@ -218,7 +241,8 @@ int fsa_cmp_topk(const void* q, const void* ck, const float* lse, int32_t dtype,
                  int64_t total_q, int64_t max_seqlen_q, int64_t max_seqlen_k,
                  int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
                  int32_t kernel_size, int32_t kernel_stride, int32_t block_size, int32_t topk,
-                 int32_t init_blocks, int32_t local_blocks, int32_t scores_to_bf16, float softmax_scale,
+                 int32_t init_blocks, int32_t local_blocks, int32_t scores_to_bf16,
+                 int32_t score_head_as_written, float softmax_scale,
                  int32_t* topk_idx, float* block_score, void* workspace, size_t workspace_bytes,
                  void* stream);
 

@@ -29,7 +29,7 @@ def test_header_symbols_are_exported_and_bound():
 
 def test_version_and_host_arithmetic():
     lib = _lib.load()
-    assert lib.fsa_version() >= 100
+    assert lib.fsa_version() >= 210
     # tiles upper bound: ceil(N*T*g / rows) + max_blocks
     assert lib.fsa_max_tiles(65536, 16, 1, 1024, 1025) == 65536 * 16 // 1024 + 1025
     # counting path (at most 4095 blocks): one count per (kv head, block or padding bucket, tile of 4096 entries)

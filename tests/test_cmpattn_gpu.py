@@ -136,6 +136,43 @@ def test_cmp_topk(dev, cu, hq, hkv, d, ks, st, bk, t, dtype):
     assert same > 0.999
 
 
+@pytest.mark.parametrize("cu,hq,hkv,d,dtype", [([0, 900, 2100], 8, 2, 128, torch.bfloat16),
+                                                ([0, 1500], 6, 2, 64, torch.float16)])
+def test_cmp_topk_score_head_as_written(dev, cu, hq, hkv, d, dtype):
+    """score_head_as_written: kv head kh is scored with q head kh (what the reference's parallel path computes,
+    nsa_ref/ops/compressed_attention.py:870, 898, 906), not with the first head kh * g of its group.  The oracle
+    gets exactly those heads as a GQA-1 problem; the default must differ from it (the heads are independent draws)."""
+    ks, st, bk, t = 32, 16, 64, 8
+    print(f"case cu={cu} hq={hq} hkv={hkv} d={d} {dtype}", flush=True)
+    q, ck, cv, do, cu_k = _make(cu, hq, hkv, d, ks, st, dtype, seed=21)
+    cu_q_t = torch.tensor(cu, dtype=torch.int32, device=dev)
+    cu_k_t = torch.tensor(cu_k, dtype=torch.int32, device=dev)
+    max_q = max(b - a for a, b in zip(cu[:-1], cu[1:]))
+    max_k = max(b - a for a, b in zip(cu_k[:-1], cu_k[1:]))
+    qd, ckd, cvd = (x.to(dev) for x in (q, ck, cv))
+    o, lse = ops.cmpattn_fwd(qd, ckd, cvd, ks, st, cu_q_t, cu_k_t, max_q)
+    got = {}
+    for aw in (False, True):
+        idx, bscore = ops.cmp_topk(qd, ckd, lse, ks, st, bk, t, cu_q_t, cu_k_t, max_q, max_k, scores_to_bf16=False,
+                                   return_block_score=True, score_head_as_written=aw)
+        torch.cuda.synchronize()
+        got[aw] = (idx.cpu(), bscore.cpu())
+        assert torch.equal(got[aw][0], orc.topk_select_ref(got[aw][1], t, cu, bk, to_bf16=False))
+    _, lse_r = orc.compressed_attention_ref(q.float(), ck.float(), cv.float(), ks, st, cu, cu_k)
+    # heads 0 .. Hkv-1 of q with their own LSE rows, one q head per kv head
+    _, bs_r = orc.compressed_topk_ref(q[:, :hkv].float(), ck.float(), lse_r[:hkv], ks, st, bk, t, cu, cu_k,
+                                      max_seqlen_q=max_q, to_bf16=False)
+    bs = got[True][1]
+    fin = ~torch.isinf(bs_r)
+    assert torch.equal(torch.isinf(bs), ~fin)
+    diff = (bs[fin] - bs_r[fin]).abs()
+    print(f"  as-written block scores: max diff {diff.max().item():.3e}", flush=True)
+    assert (diff <= 2.0 ** -6 * bs_r[fin].abs() + 2e-3).all()
+    # kv head 0 is scored by q head 0 either way; the others change
+    assert torch.equal(got[True][1][0], got[False][1][0])
+    assert not torch.allclose(got[True][1][1:][fin[1:]], got[False][1][1:][fin[1:]], atol=1e-2)
+
+
 # one case per variant of the selection kernel: block scores in 4 / 8 / 16 registers per lane (rounded to bf16),
 # fp32 scores in LDS, more than 1024 blocks in LDS
 TOPK_VARIANTS = [

@@ -99,3 +99,29 @@ def test_gate_merge(dev, dtype):
         assert torch.equal(got.cpu(), (g32[:, i, None, None] * w.float()).to(dtype))
         dg = (w.float() * x.float()).sum((1, 2))
         assert torch.allclose(d_g[:, i].float().cpu(), dg, rtol=2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d,dn", [(96, 128), (40, 64), (192, 256), (128, 96), (64, 40)])
+def test_pad_head_dim_entry_point(dev, dtype, d, dn):
+    """fsa_pad_head_dim through the C ABI: the leading columns copied bit for bit, the rest zero, on a strided
+    source (a slice of a fused projection output) - what a caller with head_dim 96 / 192 runs before and after
+    the kernels, which are built for 64 / 128 / 256 (fsa_native_head_dim names the size)."""
+    from fsa_hip import _lib
+    lib = _lib.load()
+    assert [lib.fsa_native_head_dim(x) for x in (1, 40, 64, 65, 96, 128, 129, 192, 256, 257)] == \
+        [64, 64, 64, 128, 128, 128, 256, 256, 256, -1]
+    gen = torch.Generator().manual_seed(5)
+    n, h = 777, 6
+    big = torch.randn(n, h + 2, d + 8, generator=gen).to(dtype).to(dev)
+    src = big[:, 1 : 1 + h, 4 : 4 + d]                     # strides (h + 2) * (d + 8), d + 8, 1; offset 8 bytes-aligned
+    out = torch.full((n, h, dn), 7.0, dtype=dtype, device=dev)
+    rc = lib.fsa_pad_head_dim(src.data_ptr(), src.stride(0), src.stride(1), d, out.data_ptr(), out.stride(0),
+                              out.stride(1), dn, n, h, torch.cuda.current_stream(dev).cuda_stream)
+    assert rc == 0, lib.fsa_last_error()
+    torch.cuda.synchronize()
+    m = min(d, dn)
+    assert torch.equal(out[..., :m], src[..., :m])
+    assert (out[..., m:] == 0).all()
+    # the Python layer takes the same route
+    assert torch.equal(ops._pad_d(src, dn) if dn > d else ops._cut_d(src, dn), out)
