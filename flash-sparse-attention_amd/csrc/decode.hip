@@ -549,30 +549,84 @@ static size_t dec_ws_bytes(int batch, int hq, int hkv, int d) {
 constexpr size_t DEC_STATIC_SCRATCH_BYTES = (size_t)FSA_DECODE_STATIC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char dec_static_scratch[DEC_STATIC_SCRATCH_BYTES];
 
-// Device address of the scratch array on the current device; looked up once per device.
-static int dec_static_scratch_ptr(void** out) {
-  constexpr int MAX_DEV = 64;
-  static void* ptr[MAX_DEV] = {nullptr};
-  static std::mutex mu;
+// Per-device state of the scratch array: its device address (looked up once), and the stream and completion
+// event of the last call that used it.
+struct DecStaticState {
+  void* ptr = nullptr;
+  hipEvent_t done = nullptr;
+  hipStream_t last_stream = nullptr;
+  bool used = false;
+};
+constexpr int DEC_STATIC_MAX_DEV = 64;
+static DecStaticState dec_static_state[DEC_STATIC_MAX_DEV];
+static std::mutex dec_static_mu;
+
+// Set-up for one call on `stream`: the scratch address of the current device, and - the array is shared by every
+// call on the device - an ordering edge behind the previous call when that one ran on another stream
+// (hipStreamWaitEvent on its completion event; nothing is allocated per call, the event is created once per
+// device).  Calls recorded into a graph take no part in this: a capturing stream may neither wait for nor record
+// an event of eager work, so captured calls are ordered by the graph's own dependencies.
+static int dec_static_begin(hipStream_t stream, void** out, bool* capturing) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) {
     set_error("fsa_decode_selattn_static: hipGetDevice: %s", hipGetErrorString(e));
     return (int)e;
   }
-  std::lock_guard<std::mutex> lock(mu);
-  if (dev >= 0 && dev < MAX_DEV && ptr[dev]) {
-    *out = ptr[dev];
-    return 0;
+  if (dev < 0 || dev >= DEC_STATIC_MAX_DEV) {
+    set_error("fsa_decode_selattn_static: device %d out of range", dev);
+    return FSA_ERR_UNSUPPORTED;
   }
-  void* a = nullptr;
-  e = hipGetSymbolAddress(&a, HIP_SYMBOL(dec_static_scratch));
-  if (e != hipSuccess || !a) {
-    set_error("fsa_decode_selattn_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
-    return e != hipSuccess ? (int)e : FSA_ERR_UNSUPPORTED;
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cs) != hipSuccess) {
+    (void)hipGetLastError();
+    cs = hipStreamCaptureStatusNone;
   }
-  if (dev >= 0 && dev < MAX_DEV) ptr[dev] = a;
-  *out = a;
+  *capturing = cs != hipStreamCaptureStatusNone;
+  std::lock_guard<std::mutex> lock(dec_static_mu);
+  DecStaticState& st = dec_static_state[dev];
+  if (!st.ptr) {
+    void* a = nullptr;
+    e = hipGetSymbolAddress(&a, HIP_SYMBOL(dec_static_scratch));
+    if (e != hipSuccess || !a) {
+      set_error("fsa_decode_selattn_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : FSA_ERR_UNSUPPORTED;
+    }
+    st.ptr = a;
+  }
+  *out = st.ptr;
+  if (*capturing) return 0;
+  if (!st.done) {
+    e = hipEventCreateWithFlags(&st.done, hipEventDisableTiming);
+    if (e != hipSuccess) {
+      set_error("fsa_decode_selattn_static: hipEventCreateWithFlags: %s", hipGetErrorString(e));
+      return (int)e;
+    }
+  }
+  if (st.used && st.last_stream != stream) {
+    e = hipStreamWaitEvent(stream, st.done, 0);
+    if (e != hipSuccess) {
+      set_error("fsa_decode_selattn_static: hipStreamWaitEvent: %s", hipGetErrorString(e));
+      return (int)e;
+    }
+  }
+  return 0;
+}
+
+// After the kernels of an eager call are enqueued: remember its stream and mark its end.
+static int dec_static_end(hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= DEC_STATIC_MAX_DEV) return 0;
+  std::lock_guard<std::mutex> lock(dec_static_mu);
+  DecStaticState& st = dec_static_state[dev];
+  if (!st.done) return 0;
+  hipError_t e = hipEventRecord(st.done, stream);
+  if (e != hipSuccess) {
+    set_error("fsa_decode_selattn_static: hipEventRecord: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  st.last_stream = stream;
+  st.used = true;
   return 0;
 }
 
@@ -697,11 +751,14 @@ extern "C" int fsa_decode_selattn_static(const void* q, const void* k_cache, con
     return FSA_ERR_WORKSPACE;
   }
   void* scratch = nullptr;
-  int rc = dec_static_scratch_ptr(&scratch);
+  bool capturing = false;
+  int rc = dec_static_begin((hipStream_t)stream_, &scratch, &capturing);
   if (rc) return rc;
   // every partial slot that the merge reads is written by the attention kernel of the same call: nothing in the
   // buffer has to start at zero
-  return fsa_decode_selattn(q, k_cache, v_cache, dtype, q_stride_b, q_stride_h, k_stride_n, k_stride_h, v_stride_n,
-                            v_stride_h, cu_k, seqlens, topk_idx, batch, num_q_heads, num_kv_heads, head_dim, topk, block_size,
-                            softmax_scale, o, lse, scratch, DEC_STATIC_SCRATCH_BYTES, stream_);
+  rc = fsa_decode_selattn(q, k_cache, v_cache, dtype, q_stride_b, q_stride_h, k_stride_n, k_stride_h, v_stride_n,
+                          v_stride_h, cu_k, seqlens, topk_idx, batch, num_q_heads, num_kv_heads, head_dim, topk, block_size,
+                          softmax_scale, o, lse, scratch, DEC_STATIC_SCRATCH_BYTES, stream_);
+  if (rc || capturing) return rc;
+  return dec_static_end((hipStream_t)stream_);
 }

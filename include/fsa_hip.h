@@ -327,10 +327,16 @@ int fsa_decode_selattn(const void* q, const void* k_cache, const void* v_cache, 
  * library's code object (each device the library runs on holds its copy until the
  * process ends), and the call allocates nothing.  No counterpart in the
  * reference.  Sizes with fsa_decode_workspace_bytes(...) above the buffer are
- * refused with FSA_ERR_WORKSPACE.  All calls on one device share the buffer:
- * calls that overlap on a device (different streams or threads) race; calls on
- * one stream do not.  The first call on a device looks the buffer up
- * (hipGetSymbolAddress); make it outside a stream capture. */
+ * refused with FSA_ERR_WORKSPACE.  All calls on one device share the buffer.
+ * Eager calls are kept apart by the library: a call on another stream than the
+ * previous one first waits (hipStreamWaitEvent) for that call's completion event,
+ * so consecutive calls never overlap on the buffer whatever their streams; calls
+ * issued from several threads at once are serialised only in their set-up, so
+ * give each thread's calls an order of your own.  Calls recorded into a graph
+ * take no part in that (a capturing stream cannot wait for eager work): replays
+ * that overlap other calls on the device race.  The first call on a device looks
+ * the buffer up (hipGetSymbolAddress) and creates the event; make it outside a
+ * stream capture. */
 #define FSA_DECODE_STATIC_SCRATCH_BYTES (16u << 20)
 int fsa_decode_selattn_static(const void* q, const void* k_cache, const void* v_cache, int32_t dtype,
                               int64_t q_stride_b, int64_t q_stride_h, int64_t k_stride_n, int64_t k_stride_h,

@@ -59,3 +59,57 @@ def test_static_scratch_rejects_sizes_beyond_the_buffer(dev):
         ops.decode_selattn_static(q, kc, vc, cu, idx, bk, o, lse)
     torch.cuda.synchronize()
     assert (o == 0).all() and (lse == 0).all()
+
+
+def test_static_scratch_call_can_be_recorded_into_a_graph(dev):
+    """What the entry point exists for: the call allocates nothing, so it can be recorded into a HIP graph with
+    caller-owned outputs.  After one eager call (buffer lookup), the call is captured and replayed on new query
+    values, with eager work and synchronisations between the replays; every replay must equal the eager
+    workspace entry point bit for bit.  An allocation inside the call would fail the capture."""
+    hq, hkv, d, bk, t, dtype = 8, 2, 128, 64, 16, torch.bfloat16
+    lens = [1500, 64, 700, 2999]
+    q, kc, vc, cu, idx = _inputs(lens, hq, hkv, d, bk, t, dtype, 97, dev)
+    o = torch.zeros((len(lens), hq, d), dtype=dtype, device=dev)
+    lse = torch.zeros((hq, len(lens)), dtype=torch.float32, device=dev)
+    ops.decode_selattn_static(q, kc, vc, cu, idx, bk, o, lse)          # eager first call: looks the buffer up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.decode_selattn_static(q, kc, vc, cu, idx, bk, o, lse)
+    gen = torch.Generator().manual_seed(98)
+    for rep in range(4):
+        q.copy_(torch.randn(q.shape, generator=gen).to(dtype))
+        o.fill_(float("nan"))
+        lse.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        o_ref, lse_ref = ops.decode_selattn(q, kc, vc, cu, idx, bk)     # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(o, o_ref) and torch.equal(lse, lse_ref), rep
+
+
+def test_static_scratch_calls_on_two_streams_do_not_overlap(dev):
+    """Consecutive eager calls on different streams share the one buffer: the second waits for the first's
+    completion event inside the library, so both results are exact without any synchronisation by the caller."""
+    hq, hkv, d, bk, t, dtype = 8, 2, 128, 64, 16, torch.bfloat16
+    gen = torch.Generator().manual_seed(99)
+    a_lens = torch.randint(500, 3000, (64,), generator=gen).tolist()
+    b_lens = [2000, 100]
+    ins_a = _inputs(a_lens, hq, hkv, d, bk, t, dtype, 100, dev)
+    ins_b = _inputs(b_lens, hq, hkv, d, bk, t, dtype, 101, dev)
+    ref_a = ops.decode_selattn(*ins_a, bk)
+    ref_b = ops.decode_selattn(*ins_b, bk)
+    outs = []
+    for lens in (a_lens, b_lens):
+        outs.append((torch.zeros((len(lens), hq, d), dtype=dtype, device=dev),
+                     torch.zeros((hq, len(lens)), dtype=torch.float32, device=dev)))
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(dev), torch.cuda.Stream(dev)
+    for _ in range(3):
+        with torch.cuda.stream(s1):
+            ops.decode_selattn_static(*ins_a, bk, *outs[0])
+        with torch.cuda.stream(s2):
+            ops.decode_selattn_static(*ins_b, bk, *outs[1])
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], ref_a[0]) and torch.equal(outs[0][1], ref_a[1])
+    assert torch.equal(outs[1][0], ref_b[0]) and torch.equal(outs[1][1], ref_b[1])
