@@ -69,11 +69,45 @@ def test_many_short_sequences(dev, nseq, maxlen, hkv, g, d, bk, t, dtype):
     _check(dev, nseq, cu, hkv * g, hkv, d, bk, t, dtype, both_index_paths=True)
 
 
-def _check(dev, seed, cu, hq, hkv, d, bk, t, dtype, both_index_paths=False):
+def _unforced(topk, cu, bk, seed):
+    """Lists in which the forced blocks are not a given: a third of the queries lose block 0, another third their
+    own block, and every query past its first block holds the block before its own (the layer's local_blocks = 2
+    layout) in place of one of its random picks."""
+    gen = torch.Generator().manual_seed(seed)
+    out = topk.clone()
+    hkv, n, t = out.shape
+    own = torch.cat([torch.arange(b - a) // bk for a, b in zip(cu[:-1], cu[1:])])[None, :, None]   # [1, N, 1]
+    which = torch.randint(0, 3, (hkv, n, 1), generator=gen)
+    has_prev = ((out == own - 1) & (own >= 1)).any(-1, keepdim=True)
+    # own - 1 replaces the first entry that is neither block 0, the own block nor padding
+    free = (out > 0) & (out != own) & (out != own - 1)
+    first_free = free & (free.int().cumsum(-1) == 1)
+    out = torch.where(first_free & ~has_prev & (own >= 2), (own - 1).expand_as(out).to(out.dtype), out)
+    out = torch.where((which == 0) & (out == 0) & (own >= 1), torch.full_like(out, -1), out)       # no block 0
+    out = torch.where((which == 1) & (out == own) & (own >= 1), torch.full_like(out, -1), out)     # no own block
+    return out
+
+
+@pytest.mark.parametrize("cu,hq,hkv,d,bk,t,dtype", [([0, 2100, 2164, 5000], 8, 2, 128, 64, 8, torch.bfloat16),
+                                                    ([0, 3300], 4, 4, 128, 64, 16, torch.float16)])
+def test_lists_without_forced_blocks(dev, cu, hq, hkv, d, bk, t, dtype):
+    """Nothing in the operator assumes that a query selects block 0 or its own block, or that it does not select the
+    block before its own: lists without them (and with own - 1 everywhere) against the same oracle."""
+    print(f"case cu={cu} hq={hq} hkv={hkv} d={d} bk={bk} t={t} {dtype}", flush=True)
+    topk = _unforced(make_topk_idx(cu, hkv, bk, t, seed=77), cu, bk, 78)
+    own = torch.cat([torch.arange(b - a) // bk for a, b in zip(cu[:-1], cu[1:])])[None, :, None]
+    late = (own >= 2).expand_as(topk)[..., 0]
+    assert ((topk == 0).any(-1) | ~late).float().mean() < 0.8 and ((topk == own).any(-1) | ~late).float().mean() < 0.8
+    assert ((topk == own - 1).any(-1) | ~late).all()
+    _check(dev, 5, cu, hq, hkv, d, bk, t, dtype, topk=topk)
+
+
+def _check(dev, seed, cu, hq, hkv, d, bk, t, dtype, both_index_paths=False, topk=None):
     n = cu[-1]
     std = 1.0 if dtype == torch.bfloat16 else 0.5
     q, k, v, do = make_qkv(n, hq, hkv, d, dtype, seed=100 + seed, std=std)
-    topk = _scramble(make_topk_idx(cu, hkv, bk, t, seed=200 + seed), 300 + seed)
+    if topk is None:
+        topk = _scramble(make_topk_idx(cu, hkv, bk, t, seed=200 + seed), 300 + seed)
     cu_t = torch.tensor(cu, dtype=torch.int32)
     index = ops.build_index(topk.to(dev), cu_t.to(dev), bk)
     cu_blocks, counts, starts, sel_tokens, slot_of = orc.build_index_ref(topk, cu, bk)
