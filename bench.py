@@ -80,7 +80,7 @@ def measured_traffic(workload: str):
         for label, frag in TRAFFIC_KERNEL_NAMES.items():
             if frag in m.group(1):
                 out[(label, int(m.group(2)))] = int(float(m.group(3)) * 1e9)
-    return out
+    return out, source
 
 METRIC = "selected-attn fwd+bwd ms & TFLOP/s at 64K, B_K=64, T=16, GQA 1-4; roofline %"
 
