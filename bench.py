@@ -40,24 +40,29 @@ TRAFFIC_KERNEL_NAMES = {"selattn_bwd_dqdkdv": "attn_bwd_dkdv_kernel", "selattn_f
                         "selattn_bwd_delta": "selattn_bwd_delta_kernel"}
 
 
-def csrc_sha16() -> str:
-    """Hash of the kernel sources (csrc/*.hip, csrc/*.h, the C header): identifies the code a counter summary
-    was captured from."""
+# the sources that define the kernels of the selected-attention step (index, forward, backward)
+SELATTN_SOURCES = ("fsa_common.h", "index.hip", "selattn_fwd.hip", "selattn_bwd.hip", "dkdv_kernel.h")
+
+
+def csrc_sha16(names=SELATTN_SOURCES) -> str:
+    """Hash of kernel sources under csrc/ (default: those of the selected-attention step; None: every .hip / .h):
+    identifies the code a counter summary was captured from."""
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, "flash-sparse-attention_amd", "csrc")
-    files = sorted(os.path.join(csrc, f) for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
-    files.append(os.path.join(ROOT, "include", "fsa_hip.h"))
-    for f in files:
-        h.update(os.path.basename(f).encode())
-        h.update(open(f, "rb").read())
+    if names is None:
+        names = sorted(f for f in os.listdir(csrc) if f.endswith((".hip", ".h")))
+    for f in names:
+        h.update(f.encode())
+        h.update(open(os.path.join(csrc, f), "rb").read())
     return h.hexdigest()[:16]
 
 
 def measured_traffic(workload: str):
     """({(label, gqa): bytes per launch}, source) from profiles/<summary>: lines `<kernel> grid=<n> gqa=<g> ...
-    bytes=<x> GB`.  The summary names the kernel sources it was captured from (`# csrc_sha16: <hash>`); when the
-    sources of this tree differ, nothing is returned - a stale figure is worse than none."""
+    bytes=<x> GB`.  The summary names the kernel sources it was captured from (`# csrc_sha16: <hash>` over
+    SELATTN_SOURCES); when those sources differ in this tree, nothing is returned - a stale figure is worse than
+    none."""
     import re
     out = {}
     name = TRAFFIC_FILES.get(workload, "-")

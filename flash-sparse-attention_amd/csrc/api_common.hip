@@ -45,22 +45,23 @@ pad_head_dim_kernel(const uint16_t* __restrict__ src, int64_t src_sn, int64_t sr
                     uint16_t* __restrict__ dst, int64_t dst_sn, int64_t dst_sh, int d_dst, int64_t rows,
                     int heads) {
   const int per = d_dst / 4;
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= rows * heads * per) return;
-  const int c = (int)(idx % per) * 4;
-  const int64_t rh = idx / per;
-  const int h = (int)(rh % heads);
-  const int64_t r = rh / heads;
-  const uint16_t* s = src + r * src_sn + h * src_sh + c;
-  uint2 x = make_uint2(0u, 0u);
-  if (c + 4 <= d_src) {
-    x = *reinterpret_cast<const uint2*>(s);
-  } else if (c < d_src) {  // d_src is a multiple of 4 in practice; the general tail copies element by element
-    uint16_t e[4] = {0, 0, 0, 0};
-    for (int i = 0; c + i < d_src; ++i) e[i] = s[i];
-    x = make_uint2(e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16));
+  const int64_t items = rows * heads * per;
+  for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < items; idx += (int64_t)gridDim.x * 256) {
+    const int c = (int)(idx % per) * 4;
+    const int64_t rh = idx / per;
+    const int h = (int)(rh % heads);
+    const int64_t r = rh / heads;
+    const uint16_t* s = src + r * src_sn + h * src_sh + c;
+    uint2 x = make_uint2(0u, 0u);
+    if (c + 4 <= d_src) {
+      x = *reinterpret_cast<const uint2*>(s);
+    } else if (c < d_src) {  // d_src is a multiple of 4 in practice; the general tail copies element by element
+      uint16_t e[4] = {0, 0, 0, 0};
+      for (int i = 0; c + i < d_src; ++i) e[i] = s[i];
+      x = make_uint2(e[0] | ((uint32_t)e[1] << 16), e[2] | ((uint32_t)e[3] << 16));
+    }
+    *reinterpret_cast<uint2*>(dst + r * dst_sn + h * dst_sh + c) = x;
   }
-  *reinterpret_cast<uint2*>(dst + r * dst_sn + h * dst_sh + c) = x;
 }
 }  // namespace fsa
 
@@ -79,12 +80,15 @@ extern "C" int fsa_pad_head_dim(const void* src, int64_t src_stride_n, int64_t s
   FSA_CHECK_ARG(src && dst, "fsa_pad_head_dim: null pointer");
   FSA_CHECK_ARG(rows >= 1 && heads >= 1 && d_src >= 1 && d_dst >= 4 && d_dst % 4 == 0,
                 "fsa_pad_head_dim: rows, heads and head dims must be positive, d_dst a multiple of 4");
-  FSA_CHECK_ARG((src_stride_n | src_stride_h | dst_stride_n | dst_stride_h) % 4 == 0 && ((uintptr_t)src | (uintptr_t)dst) % 8 == 0,
-                "fsa_pad_head_dim: rows must be 8-byte aligned (strides multiples of 4 elements)");
+  FSA_CHECK_ARG(src_stride_n >= 0 && src_stride_h >= 0 && dst_stride_n >= 0 && dst_stride_h >= 0 &&
+                    (src_stride_n | src_stride_h | dst_stride_n | dst_stride_h) % 4 == 0 &&
+                    ((uintptr_t)src | (uintptr_t)dst) % 8 == 0,
+                "fsa_pad_head_dim: rows must be 8-byte aligned (non-negative strides, multiples of 4 elements)");
+  FSA_CHECK_ARG(rows < ((int64_t)1 << 40) / heads / d_dst, "fsa_pad_head_dim: too many elements");
   const int64_t items = rows * heads * (d_dst / 4);
-  FSA_CHECK_ARG(items < ((int64_t)1 << 39), "fsa_pad_head_dim: too many elements");
+  const int64_t blocks = (items + 255) / 256;
   fsa::ProfScope ps_("pad_head_dim", (hipStream_t)stream_);
-  fsa::pad_head_dim_kernel<<<(unsigned)((items + 255) / 256), 256, 0, (hipStream_t)stream_>>>(
+  fsa::pad_head_dim_kernel<<<(unsigned)(blocks < (1 << 20) ? blocks : (1 << 20)), 256, 0, (hipStream_t)stream_>>>(
       (const uint16_t*)src, src_stride_n, src_stride_h, d_src, (uint16_t*)dst, dst_stride_n, dst_stride_h, d_dst,
       rows, heads);
   FSA_CHECK_LAUNCH("fsa_pad_head_dim");

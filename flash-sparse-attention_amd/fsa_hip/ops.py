@@ -42,9 +42,9 @@ def _resize_d(t: torch.Tensor, d_to: int) -> torch.Tensor:
     """[..., H, d] -> contiguous [..., H, d_to]: the leading columns copied, the rest zero (fsa_pad_head_dim)."""
     d = t.shape[-1]
     rows = t.reshape(-1, t.shape[-2], d) if t.dim() != 3 else t
-    if (t.dtype not in _DTYPE or not t.is_cuda or rows.stride(2) != 1 or d % 4 or d_to % 4
+    if (t.numel() == 0 or t.dtype not in _DTYPE or not t.is_cuda or rows.stride(2) != 1 or d % 4 or d_to % 4
             or rows.stride(0) % 4 or rows.stride(1) % 4 or t.data_ptr() % 8):
-        # shapes the C helper does not take (fp32 gradients of parameters, odd head dims): torch does the copy
+        # what the C helper does not take (empty tensors, fp32 gradients of parameters, odd head dims): torch copies
         return (torch.nn.functional.pad(t, (0, d_to - d)) if d_to > d else t[..., :d_to]).contiguous()
     out = torch.empty((*t.shape[:-1], d_to), dtype=t.dtype, device=t.device)
     o3 = out.view(-1, t.shape[-2], d_to)
