@@ -113,3 +113,22 @@ def test_every_compute_entry_point_rejects_null_pointers():
         rc = getattr(lib, name)(*vals)
         assert rc == -1, (name, rc)
         assert lib.fsa_last_error(), name
+
+
+def test_pad_head_dim_argument_checks():
+    """fsa_native_head_dim is host arithmetic; fsa_pad_head_dim refuses bad strides / alignment / sizes before any
+    launch (no device needed for either)."""
+    lib = _lib.load()
+    assert [lib.fsa_native_head_dim(d) for d in (0, 1, 64, 65, 128, 129, 256, 257)] == [-1, 64, 64, 128, 128, 256, 256, -1]
+    f = 4096
+    ok = dict(src=f, sn=96, sh=96, ds=96, dst=f, dn=128, dh=128, dd=128, rows=4, heads=1)
+
+    def call(**kw):
+        a = dict(ok, **kw)
+        return lib.fsa_pad_head_dim(a["src"], a["sn"], a["sh"], a["ds"], a["dst"], a["dn"], a["dh"], a["dd"], a["rows"],
+                                    a["heads"], None)
+
+    for bad in (dict(src=None), dict(dst=None), dict(rows=0), dict(heads=0), dict(ds=0), dict(dd=2), dict(dd=126),
+                dict(sn=-96), dict(sn=98), dict(dh=130), dict(src=f + 4), dict(rows=1 << 45)):
+        assert call(**bad) == -1, bad
+        assert b"fsa_pad_head_dim" in lib.fsa_last_error()
